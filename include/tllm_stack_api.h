@@ -1,0 +1,88 @@
+/*
+ * tllm_stack_api.h - ragged-batch step executor for decoder stacks that are described at run time.
+ *
+ * Where tllm_runtime_api.h runs one fixed network (the LLaMA decoder) on a rectangular batch, this engine runs a stack whose
+ * layers are listed in its configuration - each a token mixer of a registered kind plus an optional gated feed-forward - on a
+ * PACKED batch: a step carries, side by side, portions of prompts and single decoded tokens of several sequences.  What a
+ * sequence leaves behind lives in two stores that the caller's cache manager hands out (tensorrt_llm.runtime.KVCacheManager /
+ * StateSlotManager): pages of a block pool shared by all attention layers (one block id is valid in every layer's pool) and
+ * state slots for the recurrent layers.  The engine owns the memory, the caller owns the bookkeeping: a step names, per entry,
+ * the position of its first token, its slot and its block table.
+ *
+ * Mixer kinds: "attention" (grouped-query, `maps` attention maps per head over shared values - 2 = differential attention -,
+ * interleaved rotary positions on the first rot_dims dimensions with YaRN-style frequency scaling, tanh soft cap, per-head RMS
+ * norm of the output) and "hgrn2" (gated linear recurrence with a lower-bounded forget gate, fp32 state).  Norms are RMS norms in
+ * groups; residual updates are gated by sigmoid(W h + b); a range of layers may be run several times in a row (every pass with a
+ * cache / state of its own).
+ *
+ * Element type bfloat16: weights, activations and caches in bfloat16, fp32 accumulation, and fp32 for the residual stream, norms,
+ * scores and softmax, rotation angles, gates of a recurrence and its state.  float32: everything in fp32 with plain FMAs.
+ *
+ * Errors: NULL / non-zero + tllm_last_error().  Nothing synchronises except tllm_stack_step (it returns host results).
+ */
+#ifndef TLLM_STACK_API_H
+#define TLLM_STACK_API_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tllm_stack* tllm_stack_t;
+
+/* Configuration text, one key=value per line:
+ *   dtype (bfloat16 | float32), width, vocab, num_layers, norm_groups (1), norm_eps (1e-5), embedding_scale (1),
+ *   loop_start, loop_stop, loop_times (0, 0, 1: no loop), page_size (64), num_blocks, num_slots, debug_taps (0),
+ *   per layer i: layer.<i>.type (attention | hgrn2), .heads, .dim, .vdim, .ff (0: no feed-forward),
+ *     attention: .kv_heads, .maps (1 | 2), .diff (the constant of the second map's weight and of the output scale 1 - diff),
+ *       .scale, .softcap (0: none), .head_norm (0 | 1), .rot_dims, .rot_base, .rot_factor (0: no frequency scaling),
+ *       .rot_original, .rot_fast, .rot_slow.
+ * Weights are named l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,lq1,lk1,lq2,lk2} (attention), l<i>.mix.{q,f,f.b,lower,v,norm,o}
+ * (hgrn2), l<i>.mlp.{gate,up,down}, l<i>.rg1, l<i>.rg1.b, l<i>.rg2, l<i>.rg2.b, embed, loop.step, final.norm, head; linear
+ * weights [out, in]. */
+tllm_stack_t tllm_stack_create(const char* config_text);
+
+/* One weight tensor from HOST memory; dtype 0 = fp32, 7 = bfloat16 (nvinfer1::DataType codes).  Converted to the engine's element
+ * type on the way in. */
+int32_t tllm_stack_set_tensor(tllm_stack_t s, const char* name, int32_t dtype, const int64_t* dims, int32_t nbDims, const void* data);
+
+/* Resolves the weights against the configuration (names the first missing / mis-shaped one), fuses the projections that share an
+ * input, allocates block pools and state slots. */
+int32_t tllm_stack_finalize(tllm_stack_t s);
+
+typedef struct
+{
+    int32_t n_tokens, n_entries, n_want, max_blocks;
+    const int32_t* tokens;      /* [n_tokens] ids, entries back to back */
+    const int32_t* ent_count;   /* [n_entries] tokens of each entry (>= 1) */
+    const int32_t* ent_pos0;    /* [n_entries] position of the entry's first token in its sequence (0: a new sequence) */
+    const int32_t* ent_slot;    /* [n_entries] state slot of the sequence */
+    const int32_t* block_table; /* [n_entries, max_blocks] block ids of the sequence, in order */
+    const int32_t* want_rows;   /* [n_want] rows of the packed batch whose logits are asked for */
+} tllm_stack_batch_t;
+
+/* Runs one step.  logits_out: host fp32 [n_want, vocab] or NULL; next_ids_out: host int32 [n_want] (arg-max of each wanted row, the
+ * greedy sampler) or NULL.  Every index is checked on the host before anything is launched. */
+int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* batch, float* logits_out, int32_t* next_ids_out, void* stream);
+
+/* Geometry the cache manager needs. */
+int32_t tllm_stack_page_size(tllm_stack_t s);
+int32_t tllm_stack_num_blocks(tllm_stack_t s);
+int32_t tllm_stack_num_slots(tllm_stack_t s);
+int32_t tllm_stack_vocab(tllm_stack_t s);
+int32_t tllm_stack_layer_runs(tllm_stack_t s); /* layers as executed, a looped layer counted once per pass */
+int64_t tllm_stack_weight_bytes(tllm_stack_t s);
+/* bytes one step moves at least: weights once, plus the cache / state the given contexts touch (roofline denominators) */
+int64_t tllm_stack_step_bytes(tllm_stack_t s, int32_t n_tokens, int64_t context_tokens, int32_t n_entries);
+
+/* debug_taps=1: the residual stream behind layer run `run` of the last step, fp32 [n_tokens, width], to host memory. */
+int32_t tllm_stack_get_tap(tllm_stack_t s, int32_t run, float* out, size_t n_floats);
+
+void tllm_stack_destroy(tllm_stack_t s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -39,6 +39,20 @@ __device__ __forceinline__ int32_t f2i32_rni_sat(float x)
     return (int32_t) r;
 }
 
+// bfloat16 <-> fp32: the upper half of the fp32 pattern; to bfloat16 with round-to-nearest-even (NaN stays NaN)
+__device__ __forceinline__ float bf2f(uint16_t bits)
+{
+    return __builtin_bit_cast(float, (uint32_t) bits << 16);
+}
+
+__device__ __forceinline__ uint16_t f2bf(float f)
+{
+    const uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u)
+        return (uint16_t) ((u >> 16) | 0x40u);
+    return (uint16_t) ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
 __device__ __forceinline__ float h2f(uint16_t bits)
 {
     _Float16 h;

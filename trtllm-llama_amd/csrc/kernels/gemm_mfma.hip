@@ -4,6 +4,8 @@
 //               (A10: K/cutlass_kernels/int8_gemm/int8_gemm_template.h:56-172 + epilogue_per_row_per_col_scale.h:279-347)
 //   W_FP16      A fp16, W fp16       v_mfma_f32_32x32x16_f16, fp32 accumulate          (A7: P/gemmPlugin, cuBLAS fp16/fp32)
 //   W_INT8_WOQ  A fp16, W u8 = q+128 dequantised to fp16 while staging, fp16 MFMA, * s[n] in the epilogue
+//   W_BF16      A bf16, W bf16       v_mfma_f32_32x32x16_bf16, fp32 accumulate; bf16 / fp32 output or the gated fp32
+//               residual update of the stack engine (stack_kernels.h)
 //   W_INT4_WOQ  A fp16, W nibbles   (A8: K/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h:60-160)
 //
 // One workgroup of 4 waves computes a 128 x 128 tile of C; every wave owns a 64 x 64 quadrant = 2 x 2 MFMA tiles of
@@ -29,6 +31,7 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int BM = 128, BN = 128, BKB = 64; // BKB: bytes of K per operand row per slab (in the LDS image)
 
@@ -100,7 +103,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
             if (m0 + r < M && kb < K * A_ES)
                 ra[h] = *reinterpret_cast<const uint4*>(a_base + ((int64_t) (m0 + r) * p.lda) * A_ES + kb);
         }
-        if constexpr (WT == W_INT8_SQ || WT == W_FP16)
+        if constexpr (WT == W_INT8_SQ || WT == W_FP16 || WT == W_BF16)
         {
 #pragma unroll
             for (int h = 0; h < 2; ++h)
@@ -136,7 +139,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
             *reinterpret_cast<uint4*>(As + swz(lr + h * 64, lc)) = ra[h];
-        if constexpr (WT == W_INT8_SQ || WT == W_FP16)
+        if constexpr (WT == W_INT8_SQ || WT == W_FP16 || WT == W_BF16)
         {
 #pragma unroll
             for (int h = 0; h < 2; ++h)
@@ -204,6 +207,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
                         const i32x4 b4 = {(int) bf[j].x, (int) bf[j].y, (int) bf[j].z, (int) bf[j].w};
                         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, b4, acc[i][j], 0, 0, 0);
                     }
+                    else if constexpr (WT == W_BF16)
+                    {
+                        bf16x8 a8, b8;
+                        __builtin_memcpy(&a8, &af[i], 16);
+                        __builtin_memcpy(&b8, &bf[j], 16);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a8, b8, acc[i][j], 0, 0, 0);
+                    }
                     else
                     {
                         f16x8 a8, b8;
@@ -256,6 +266,25 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
                             reinterpret_cast<float*>(p.c)[o] = v;
                     }
                 }
+                else if constexpr (WT == W_BF16)
+                {
+                    const float v = acc[i][j][r];
+                    if (p.resid)
+                    {
+                        float g = 1.f;
+                        if (p.gate)
+                        {
+                            const float z = bf2f(reinterpret_cast<const uint16_t*>(p.gate)[(int64_t) row * p.ldg + col])
+                                + (p.gate_bias ? p.gate_bias[col] : 0.f);
+                            g = 1.f / (1.f + expf(-z));
+                        }
+                        p.resid[(int64_t) row * p.ldr + col] += g * v;
+                    }
+                    else if (p.out_dtype == DT_BFLOAT16)
+                        reinterpret_cast<uint16_t*>(p.c)[o] = f2bf(v);
+                    else
+                        reinterpret_cast<float*>(p.c)[o] = v;
+                }
                 else
                 {
                     const float v = acc[i][j][r] * sc;
@@ -301,12 +330,15 @@ int launch_gemm_mfma(const GemmParams& p, hipStream_t stream)
         return 1;
     if (!sq && p.out_dtype == DT_INT32)
         return 1;
+    if (p.wtype == W_BF16 ? (p.out_dtype != DT_BFLOAT16 && p.out_dtype != DT_FLOAT) : p.out_dtype == DT_BFLOAT16)
+        return 1;
     switch (p.wtype)
     {
     case W_FP16: return launch_wt<W_FP16>(p, stream);
     case W_INT8_WOQ: return launch_wt<W_INT8_WOQ>(p, stream);
     case W_INT4_WOQ: return launch_wt<W_INT4_WOQ>(p, stream);
     case W_INT8_SQ: return launch_wt<W_INT8_SQ>(p, stream);
+    case W_BF16: return launch_wt<W_BF16>(p, stream);
     default: return 1;
     }
 }

@@ -21,7 +21,8 @@ enum DType : int32_t
     DT_FLOAT = 0,
     DT_HALF = 1,
     DT_INT8 = 2,
-    DT_INT32 = 3
+    DT_INT32 = 3,
+    DT_BFLOAT16 = 7 // nvinfer1::DataType::kBF16 (W_BF16 products only)
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -35,7 +36,8 @@ enum WType : int32_t
     W_FP16 = 0,     // W fp16 [N, K] row-major
     W_INT8_WOQ = 1, // W u8 = q + 128, [N, ldw] (k contiguous), fp16 per-column scales; x fp16
     W_INT4_WOQ = 2, // W packed nibbles n = q + 8, see weight_layout.h; fp16 per-column scales; x fp16
-    W_INT8_SQ = 3   // W s8 [N, ldw]; x s8; int32 accumulate; fp32 per-row x per-col scales
+    W_INT8_SQ = 3,  // W s8 [N, ldw]; x s8; int32 accumulate; fp32 per-row x per-col scales
+    W_BF16 = 4      // W bfloat16 [N, K] row-major; x bfloat16 (MFMA GEMM only: the stack engine's products, stack_kernels.h)
 };
 
 enum Prologue : int32_t
@@ -350,6 +352,13 @@ struct GemmParams
     const void* scale_col2 = nullptr;
     const float* scale_row2 = nullptr; // static dequantisation scale of the second GEMM [1] (null: scale_row)
     const float* swiglu_qscale = nullptr;
+    // W_BF16 only (the stack engine's layer seam): when set, nothing is written to c and
+    //   resid[m, n] += sigmoid(gate[m, n] + gate_bias[n]) * gemm   (fp32 [M, ldr]; gate bfloat16 [M, ldg] or null: plain += )
+    float* resid = nullptr;
+    int64_t ldr = 0;
+    const void* gate = nullptr;
+    int64_t ldg = 0;
+    const float* gate_bias = nullptr;
     // microbench hook (tllm_gemm_set_clock_probe), set by the launchers only: 2 x uint64 per workgroup {shader cycles, 100 MHz ticks}
     void* clock_probe = nullptr;
     // split-K-2 forms of gemm_sqp.hip (r06), set by the launcher only: per tile two slabs of AH x BN accumulators + two flag words

@@ -1,0 +1,232 @@
+// Products of the stack engine (stack_kernels.h): C[m,n] = sum_k A[m,k] * W[n,k] with the layer seam in the epilogue.
+//
+//   bfloat16, M > 8 : MFMA tiles of gemm_mfma.hip (v_mfma_f32_32x32x16_bf16);
+//   bfloat16, M <= 8: skinny_kernel below - HBM-bound, a wave streams R weight rows with 16-byte non-temporal loads and keeps the
+//                     M activation rows' chunks in registers; fp32 accumulation, DPP reduction;
+//   float32         : fma_tile_kernel - 64 x 64 tiles of plain fp32 FMAs through LDS (no reduced-precision matrix mode), any shape;
+//                     also the fallback for bfloat16 operands whose rows are not 16-byte aligned.
+#include "dev_utils.h"
+#include "stack_kernels.h"
+
+namespace tllm
+{
+namespace kernels
+{
+int launch_gemm_mfma(const GemmParams& p, hipStream_t stream); // gemm_mfma.hip; 1: shape not served
+
+using namespace dev;
+
+namespace
+{
+
+template <int DT>
+__device__ __forceinline__ float ld_el(const void* p, int64_t i)
+{
+    if constexpr (DT == DT_BF16)
+        return bf2f(reinterpret_cast<const uint16_t*>(p)[i]);
+    else
+        return reinterpret_cast<const float*>(p)[i];
+}
+
+template <int DT>
+__device__ __forceinline__ void seam(const StackGemmParams& p, int row, int col, float v)
+{
+    if (p.resid)
+    {
+        float g = 1.f;
+        if (p.gate)
+        {
+            const float z = ld_el<DT>(p.gate, (int64_t) row * p.ldg + col) + (p.gate_bias ? p.gate_bias[col] : 0.f);
+            g = 1.f / (1.f + expf(-z));
+        }
+        p.resid[(int64_t) row * p.ldr + col] += g * v;
+    }
+    else if (p.out_f32 || DT == DT_FLOAT)
+        reinterpret_cast<float*>(p.c)[(int64_t) row * p.ldc + col] = v;
+    else
+        reinterpret_cast<uint16_t*>(p.c)[(int64_t) row * p.ldc + col] = f2bf(v);
+}
+
+constexpr int TM = 64, TN = 64, TK = 16;
+
+template <int DT>
+__global__ __launch_bounds__(256) void fma_tile_kernel(const StackGemmParams p)
+{
+    __shared__ float As[TK][TM + 4];
+    __shared__ float Ws[TK][TN + 4];
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            acc[i][j] = 0.f;
+    for (int k0 = 0; k0 < p.K; k0 += TK)
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            const int idx = tid + i * 256, r = idx / TK, k = idx % TK;
+            As[k][r] = (m0 + r < p.M && k0 + k < p.K) ? ld_el<DT>(p.a, (int64_t) (m0 + r) * p.lda + k0 + k) : 0.f;
+            Ws[k][r] = (n0 + r < p.N && k0 + k < p.K) ? ld_el<DT>(p.w, (int64_t) (n0 + r) * p.K + k0 + k) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < TK; ++k)
+        {
+            float a[4], w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                a[i] = As[k][ty * 4 + i];
+                w[i] = Ws[k][tx * 4 + i];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const int row = m0 + ty * 4 + i, col = n0 + tx * 4 + j;
+            if (row < p.M && col < p.N)
+                seam<DT>(p, row, col, acc[i][j]);
+        }
+}
+
+// bfloat16, M <= MR rows: 4 waves per workgroup, R weight rows per wave
+constexpr int SK_R = 2;
+
+template <int MR>
+__global__ __launch_bounds__(256) void skinny_kernel(const StackGemmParams p)
+{
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int n0 = (blockIdx.x * 4 + wid) * SK_R;
+    if (n0 >= p.N)
+        return;
+    float acc[SK_R][MR];
+#pragma unroll
+    for (int r = 0; r < SK_R; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+            acc[r][m] = 0.f;
+    const uint16_t* a = reinterpret_cast<const uint16_t*>(p.a);
+    const uint16_t* w = reinterpret_cast<const uint16_t*>(p.w);
+    for (int k = lane * 8; k < p.K; k += 64 * 8)
+    {
+        uint4 wv[SK_R];
+#pragma unroll
+        for (int r = 0; r < SK_R; ++r)
+            wv[r] = n0 + r < p.N ? ld_nt16(w + (int64_t) (n0 + r) * p.K + k) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+        {
+            if (m >= p.M)
+                break;
+            const uint4 xv = *reinterpret_cast<const uint4*>(a + (int64_t) m * p.lda + k);
+            const uint32_t xs[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+            for (int r = 0; r < SK_R; ++r)
+            {
+                const uint32_t ws[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    acc[r][m] = fmaf(__builtin_bit_cast(float, xs[i] << 16), __builtin_bit_cast(float, ws[i] << 16), acc[r][m]);
+                    acc[r][m] = fmaf(__builtin_bit_cast(float, xs[i] & 0xffff0000u), __builtin_bit_cast(float, ws[i] & 0xffff0000u), acc[r][m]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < SK_R; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+        {
+            const float s = wave_sum(acc[r][m]);
+            if (lane == 0 && m < p.M && n0 + r < p.N)
+                seam<DT_BF16>(p, m, n0 + r, s);
+        }
+}
+
+inline int launched(const char* what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+    {
+        set_error("%s launch failed: %s", what, hipGetErrorString(e));
+        return -1;
+    }
+    return 0;
+}
+
+} // namespace
+
+int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
+{
+    if (p.M <= 0 || p.N <= 0)
+        return 0;
+    if (p.K <= 0 || !p.a || !p.w || (!p.c && !p.resid))
+    {
+        set_error("stack_gemm: M %d N %d K %d with a missing operand", p.M, p.N, p.K);
+        return -1;
+    }
+    if (p.dtype != DT_BF16 && p.dtype != DT_FLOAT)
+    {
+        set_error("stack_gemm: element type %d is not served (bfloat16 or float32)", p.dtype);
+        return -1;
+    }
+    const dim3 tiles((p.N + TN - 1) / TN, (p.M + TM - 1) / TM);
+    if (p.dtype == DT_FLOAT)
+    {
+        hipLaunchKernelGGL((fma_tile_kernel<DT_FLOAT>), tiles, dim3(256), 0, stream, p);
+        return launched("stack_gemm fp32");
+    }
+    const bool aligned = !(reinterpret_cast<uintptr_t>(p.a) & 15) && !(reinterpret_cast<uintptr_t>(p.w) & 15) && p.K % 8 == 0 && p.lda % 8 == 0;
+    if (aligned && p.M <= 8)
+    {
+        const dim3 grid((p.N + 4 * SK_R - 1) / (4 * SK_R));
+        if (p.M <= 1)
+            hipLaunchKernelGGL((skinny_kernel<1>), grid, dim3(256), 0, stream, p);
+        else if (p.M <= 4)
+            hipLaunchKernelGGL((skinny_kernel<4>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((skinny_kernel<8>), grid, dim3(256), 0, stream, p);
+        return launched("stack_gemm skinny");
+    }
+    if (aligned)
+    {
+        GemmParams g;
+        g.wtype = W_BF16;
+        g.out_dtype = p.out_f32 ? DT_FLOAT : DT_BFLOAT16;
+        g.M = p.M;
+        g.N = p.N;
+        g.K = p.K;
+        g.a = p.a;
+        g.lda = p.lda;
+        g.w = p.w;
+        g.ldw = (int64_t) p.K * 2;
+        g.c = p.c;
+        g.ldc = p.ldc;
+        g.resid = p.resid;
+        g.ldr = p.ldr;
+        g.gate = p.gate;
+        g.ldg = p.ldg;
+        g.gate_bias = p.gate_bias;
+        const int rc = launch_gemm_mfma(g, stream);
+        if (rc <= 0)
+            return rc;
+    }
+    hipLaunchKernelGGL((fma_tile_kernel<DT_BF16>), tiles, dim3(256), 0, stream, p);
+    return launched("stack_gemm bf16 fma tiles");
+}
+
+} // namespace kernels
+} // namespace tllm

@@ -1,0 +1,585 @@
+// Pointwise, rotary / cache-append, general attention and HGRN2 kernels of the ragged-batch stack engine (stack_kernels.h).
+// Everything that a norm, a softmax, a recurrence or the residual stream touches is fp32; `DT` is the storage type of
+// activations, weights and caches (bfloat16 or fp32).
+#include "dev_utils.h"
+#include "stack_kernels.h"
+#include <cmath>
+#include <vector>
+
+namespace tllm
+{
+namespace kernels
+{
+using namespace dev;
+
+namespace
+{
+
+template <int DT>
+struct El;
+template <>
+struct El<DT_FLOAT>
+{
+    typedef float type;
+    static __device__ __forceinline__ float ld(const void* p, int64_t i)
+    {
+        return reinterpret_cast<const float*>(p)[i];
+    }
+    static __device__ __forceinline__ void st(void* p, int64_t i, float v)
+    {
+        reinterpret_cast<float*>(p)[i] = v;
+    }
+};
+template <>
+struct El<DT_BF16>
+{
+    typedef uint16_t type;
+    static __device__ __forceinline__ float ld(const void* p, int64_t i)
+    {
+        return bf2f(reinterpret_cast<const uint16_t*>(p)[i]);
+    }
+    static __device__ __forceinline__ void st(void* p, int64_t i, float v)
+    {
+        reinterpret_cast<uint16_t*>(p)[i] = f2bf(v);
+    }
+};
+
+inline int launched(const char* what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+    {
+        set_error("%s launch failed: %s", what, hipGetErrorString(e));
+        return -1;
+    }
+    return 0;
+}
+
+inline bool known_dtype(int32_t dt, const char* what)
+{
+    if (dt == DT_BF16 || dt == DT_FLOAT)
+        return true;
+    set_error("%s: element type %d is not served (bfloat16 or float32)", what, dt);
+    return false;
+}
+
+// ------------------------------------------------------------------------------------------------------------ pointwise
+template <int DT>
+__global__ __launch_bounds__(256) void embed_kernel(float* x, float* keep, const int32_t* ids, const void* table, int width, int vocab,
+    float scale)
+{
+    const int t = blockIdx.x;
+    int id = ids[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    for (int c = threadIdx.x; c < width; c += blockDim.x)
+    {
+        const float v = El<DT>::ld(table, (int64_t) id * width + c) * scale;
+        x[(int64_t) t * width + c] = v;
+        if (keep)
+            keep[(int64_t) t * width + c] = v;
+    }
+}
+
+__global__ __launch_bounds__(256) void pass_entry_kernel(float* x, const float* add, const float* row, int64_t n, int width)
+{
+    const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n)
+        return;
+    float v = x[i];
+    if (add)
+        v += add[i];
+    if (row)
+        v += row[i % width];
+    x[i] = v;
+}
+
+// one workgroup per row, wave w takes groups w, w + waves, ...: no workgroup barrier
+template <int DT>
+__global__ __launch_bounds__(256) void group_rmsnorm_kernel(void* y1, void* y2, const float* x, const int32_t* rows, const float* w1,
+    const float* w2, int width, int groups, float eps)
+{
+    const int r = blockIdx.x;
+    const float* xr = x + (int64_t) (rows ? rows[r] : r) * width;
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int gs = width / groups;
+    for (int g = wid; g < groups; g += nw)
+    {
+        const float* xg = xr + g * gs;
+        float ss = 0.f;
+        for (int i = lane; i < gs; i += 64)
+            ss += xg[i] * xg[i];
+        ss = wave_sum(ss);
+        const float inv = 1.f / sqrtf(ss / (float) gs + eps);
+        for (int i = lane; i < gs; i += 64)
+        {
+            const int c = g * gs + i;
+            const float n = xg[i] * inv;
+            El<DT>::st(y1, (int64_t) r * width + c, n * w1[c]);
+            if (y2)
+                El<DT>::st(y2, (int64_t) r * width + c, n * w2[c]);
+        }
+    }
+}
+
+__device__ __forceinline__ float gelu_tanh(float z)
+{
+    return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void gelu_gate_kernel(void* y, const void* gu, int tokens, int ff, int64_t ld)
+{
+    const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t) tokens * ff)
+        return;
+    const int t = (int) (i / ff), c = (int) (i % ff);
+    const float g = El<DT>::ld(gu, (int64_t) t * ld + c), u = El<DT>::ld(gu, (int64_t) t * ld + ff + c);
+    float a = gelu_tanh(g);
+    if (DT == DT_BF16)
+        a = bf2f(f2bf(a)); // the activation is a bfloat16 value before it meets the other branch
+    El<DT>::st(y, i, a * u);
+}
+
+// --------------------------------------------------------------------------------------------------- rotary + cache append
+template <int DT>
+__global__ __launch_bounds__(256) void rope_kv_kernel(const StackAttnParams p)
+{
+    const int t = blockIdx.x;
+    const int e = p.tok_entry[t], pos = p.tok_pos[t];
+    const int blk = p.block_table[(int64_t) e * p.max_blocks + pos / p.page], off = pos % p.page;
+    const int D = p.dim, nq = p.heads * p.maps * D, nk = p.kv_heads * p.maps * D, nv = p.kv_heads * p.vdim;
+    const int64_t row = (int64_t) t * p.ldp;
+    for (int i = threadIdx.x; i < nq + nk; i += blockDim.x)
+    {
+        const int d = i % D;
+        float v = El<DT>::ld(p.proj, row + i);
+        if (d < p.rot_dims)
+        {
+            const float other = El<DT>::ld(p.proj, row + (i ^ 1)); // pairs (2i, 2i + 1): D is even, so is every map's start
+            const float a = (float) pos * p.freq[d >> 1];
+            float sn, cs;
+            sincosf(a, &sn, &cs);
+            sn *= p.mscale;
+            cs *= p.mscale;
+            v = (d & 1) ? v * cs + other * sn : v * cs - other * sn;
+        }
+        if (i < nq)
+            El<DT>::st(p.q, (int64_t) t * nq + i, v);
+        else
+        {
+            const int j = i - nq, gm = j / D; // gm = kv head * maps + map
+            El<DT>::st(p.k_pool, (((int64_t) blk * (p.kv_heads * p.maps) + gm) * p.page + off) * D + d, v);
+        }
+    }
+    for (int i = threadIdx.x; i < nv; i += blockDim.x)
+    {
+        const int g = i / p.vdim, c = i % p.vdim;
+        El<DT>::st(p.v_pool, (((int64_t) blk * p.kv_heads + g) * p.page + off) * p.vdim + c, El<DT>::ld(p.proj, row + nq + nk + i));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ attention, general form
+// One workgroup per (row, head): scores of 128 keys at a time by one thread per key, online softmax per map, P V by one thread
+// per value channel.  Any dim / vdim <= 512, both element types; the tiled kernels of stack_attn.hip take the shapes they serve.
+constexpr int AT = 128, A_CPT = 4;
+
+template <int DT, int MAPS>
+__global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams p)
+{
+    extern __shared__ float sm[];
+    float* qs = sm;                      // [MAPS][dim]
+    float* ps = qs + MAPS * p.dim;       // [MAPS][AT]
+    float* red = ps + MAPS * AT;         // [32]
+    __shared__ int blk_of[AT];
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int e = p.tok_entry[t], pos = p.tok_pos[t];
+    const int g = h / (p.heads / p.kv_heads), D = p.dim, V = p.vdim;
+    const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
+    for (int i = tid; i < MAPS * D; i += AT)
+        qs[i] = El<DT>::ld(p.q, ((int64_t) t * p.heads + h) * MAPS * D + i);
+    float m_run[MAPS], l_run[MAPS], acc[MAPS][A_CPT];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+    {
+        m_run[m] = -INFINITY;
+        l_run[m] = 0.f;
+#pragma unroll
+        for (int c = 0; c < A_CPT; ++c)
+            acc[m][c] = 0.f;
+    }
+    __syncthreads();
+    const int nkeys = pos + 1;
+    for (int k0 = 0; k0 < nkeys; k0 += AT)
+    {
+        const int kj = k0 + tid;
+        float s[MAPS];
+        int blk = 0;
+        if (kj < nkeys)
+        {
+            blk = table[kj / p.page];
+            const int off = kj % p.page;
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m)
+            {
+                const int64_t kb = (((int64_t) blk * (p.kv_heads * MAPS) + g * MAPS + m) * p.page + off) * D;
+                float a = 0.f;
+                for (int d = 0; d < D; ++d)
+                    a += qs[m * D + d] * El<DT>::ld(p.k_pool, kb + d);
+                a *= p.scale;
+                if (p.softcap > 0.f)
+                    a = p.softcap * tanhf(a / p.softcap);
+                s[m] = a;
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m)
+                s[m] = -INFINITY;
+        }
+        blk_of[tid] = blk;
+        float corr[MAPS];
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m)
+        {
+            const float bm = block_max(s[m], red);
+            const float mn = fmaxf(m_run[m], bm);
+            corr[m] = expf(m_run[m] - mn); // 0 at the first block
+            const float pj = kj < nkeys ? expf(s[m] - mn) : 0.f;
+            ps[m * AT + tid] = pj;
+            const float bs = block_sum(pj, red);
+            l_run[m] = l_run[m] * corr[m] + bs;
+            m_run[m] = mn;
+        }
+        __syncthreads();
+        const int nb = nkeys - k0 < AT ? nkeys - k0 : AT;
+#pragma unroll
+        for (int c = 0; c < A_CPT; ++c)
+        {
+            const int ch = tid + c * AT;
+            if (ch >= V)
+                break;
+            float a[MAPS];
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m)
+                a[m] = acc[m][c] * corr[m];
+            for (int j = 0; j < nb; ++j)
+            {
+                const float v = El<DT>::ld(p.v_pool, (((int64_t) blk_of[j] * p.kv_heads + g) * p.page + (k0 + j) % p.page) * V + ch);
+#pragma unroll
+                for (int m = 0; m < MAPS; ++m)
+                    a[m] += ps[m * AT + j] * v;
+            }
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m)
+                acc[m][c] = a[m];
+        }
+        __syncthreads();
+    }
+    float o[A_CPT], ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < A_CPT; ++c)
+    {
+        o[c] = 0.f;
+        if (tid + c * AT < V)
+        {
+            o[c] = acc[0][c] / l_run[0];
+            if (MAPS == 2)
+                o[c] -= p.lambda * (acc[MAPS - 1][c] / l_run[MAPS - 1]);
+            ss += o[c] * o[c];
+        }
+    }
+    float mul = 1.f;
+    if (p.head_norm)
+    {
+        ss = block_sum(ss, red);
+        mul = p.out_scale / sqrtf(ss / (float) V + p.eps);
+    }
+#pragma unroll
+    for (int c = 0; c < A_CPT; ++c)
+        if (tid + c * AT < V)
+            El<DT>::st(p.out, ((int64_t) t * p.heads + h) * V + tid + c * AT, o[c] * mul);
+}
+
+// ------------------------------------------------------------------------------------------------------------------ HGRN2
+// One wave per (entry, head, 64 value channels): lane v keeps column S[:, v] in registers and walks the entry's rows in
+// order; the row's q and forget gate are computed once per (row, channel of dim) by the lanes and shared through LDS, HC rows
+// at a time.  No cross-lane traffic in the recurrence itself.
+constexpr int HC = 8;
+
+template <int DT, int DMAX>
+__global__ __launch_bounds__(64) void hgrn2_scan_kernel(const StackHgrnParams p)
+{
+    __shared__ float qf[HC][2][DMAX];
+    const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int v = blockIdx.z * 64 + lane;
+    const int D = p.dim, V = p.vdim, HD = p.heads * D;
+    const int first = p.ent_first[e], count = p.ent_count[e];
+    const bool live = v < V;
+    float* sp = p.state + (((int64_t) p.ent_slot[e] * p.heads + h) * D) * V + v;
+    float S[DMAX];
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d)
+        S[d] = (live && d < D && p.ent_pos0[e] > 0) ? sp[(int64_t) d * V] : 0.f;
+    for (int t0 = 0; t0 < count; t0 += HC)
+    {
+        const int nt = count - t0 < HC ? count - t0 : HC;
+        __syncthreads();
+        for (int i = lane; i < nt * D; i += 64)
+        {
+            const int tt = i / D, d = i % D;
+            const int64_t row = (int64_t) (first + t0 + tt) * p.ldp;
+            float qr = El<DT>::ld(p.proj, row + h * D + d);
+            qr = qr / (1.f + expf(-qr));
+            if (DT == DT_BF16)
+                qr = bf2f(f2bf(qr)); // the projection's activation is a bfloat16 value; everything behind it is fp32
+            const float fr = El<DT>::ld(p.proj, row + HD + h * D + d) + p.f_bias[h * D + d];
+            const float lo = p.lower[h * D + d];
+            qf[tt][0][d] = qr;
+            qf[tt][1][d] = lo + (1.f - lo) * (1.f / (1.f + expf(-fr)));
+        }
+        __syncthreads();
+        if (live)
+        {
+            for (int tt = 0; tt < nt; ++tt)
+            {
+                const int64_t r = first + t0 + tt;
+                const float vv = El<DT>::ld(p.proj, r * p.ldp + 2 * HD + h * V + v);
+                float o = 0.f;
+#pragma unroll
+                for (int d = 0; d < DMAX; ++d)
+                {
+                    if (d < D)
+                    {
+                        const float f = qf[tt][1][d];
+                        S[d] = f * S[d] + (1.f - f) * vv;
+                        o += S[d] * qf[tt][0][d];
+                    }
+                }
+                p.o32[r * (p.heads * V) + h * V + v] = o;
+            }
+        }
+    }
+    if (live)
+    {
+#pragma unroll
+        for (int d = 0; d < DMAX; ++d)
+            if (d < D)
+                sp[(int64_t) d * V] = S[d];
+    }
+}
+
+// per (row, head): o / sqrt(mean(o^2) + eps) * w over the head's vdim channels; one wave each
+template <int DT>
+__global__ __launch_bounds__(256) void head_rmsnorm_kernel(void* y, const float* o, const float* w, int64_t n_heads_total, int vdim, float eps)
+{
+    const int64_t i = (int64_t) blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (i >= n_heads_total)
+        return;
+    const float* oi = o + i * vdim;
+    float ss = 0.f;
+    for (int c = lane; c < vdim; c += 64)
+        ss += oi[c] * oi[c];
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float) vdim + eps);
+    for (int c = lane; c < vdim; c += 64)
+        El<DT>::st(y, i * vdim + c, oi[c] * inv * w[c]);
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------------------------------------------- launchers
+int launch_stack_embed(float* x, float* keep, const int32_t* ids, const void* table, int32_t dtype, int32_t tokens, int32_t width,
+    int32_t vocab, float scale, hipStream_t stream)
+{
+    if (tokens <= 0)
+        return 0;
+    if (!known_dtype(dtype, "stack_embed"))
+        return -1;
+    if (dtype == DT_BF16)
+        hipLaunchKernelGGL((embed_kernel<DT_BF16>), dim3(tokens), dim3(256), 0, stream, x, keep, ids, table, width, vocab, scale);
+    else
+        hipLaunchKernelGGL((embed_kernel<DT_FLOAT>), dim3(tokens), dim3(256), 0, stream, x, keep, ids, table, width, vocab, scale);
+    return launched("stack_embed");
+}
+
+int launch_stack_pass_entry(float* x, const float* add, const float* row, int32_t tokens, int32_t width, hipStream_t stream)
+{
+    const int64_t n = (int64_t) tokens * width;
+    if (n <= 0 || (!add && !row))
+        return 0;
+    hipLaunchKernelGGL(pass_entry_kernel, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, stream, x, add, row, n, width);
+    return launched("stack_pass_entry");
+}
+
+int launch_stack_group_rmsnorm(void* y1, void* y2, const float* x, const int32_t* rows, const float* w1, const float* w2, int32_t dtype,
+    int32_t n_rows, int32_t width, int32_t groups, float eps, hipStream_t stream)
+{
+    if (n_rows <= 0)
+        return 0;
+    if (!known_dtype(dtype, "stack_group_rmsnorm"))
+        return -1;
+    if (groups < 1 || width % groups)
+    {
+        set_error("stack_group_rmsnorm: width %d does not split into %d equal groups", width, groups);
+        return -1;
+    }
+    if (dtype == DT_BF16)
+        hipLaunchKernelGGL((group_rmsnorm_kernel<DT_BF16>), dim3(n_rows), dim3(256), 0, stream, y1, y2, x, rows, w1, w2, width, groups, eps);
+    else
+        hipLaunchKernelGGL((group_rmsnorm_kernel<DT_FLOAT>), dim3(n_rows), dim3(256), 0, stream, y1, y2, x, rows, w1, w2, width, groups, eps);
+    return launched("stack_group_rmsnorm");
+}
+
+int launch_stack_gelu_gate(void* y, const void* gu, int32_t dtype, int32_t tokens, int32_t ff, int64_t ld, hipStream_t stream)
+{
+    const int64_t n = (int64_t) tokens * ff;
+    if (n <= 0)
+        return 0;
+    if (!known_dtype(dtype, "stack_gelu_gate"))
+        return -1;
+    const dim3 grid((unsigned) ((n + 255) / 256));
+    if (dtype == DT_BF16)
+        hipLaunchKernelGGL((gelu_gate_kernel<DT_BF16>), grid, dim3(256), 0, stream, y, gu, tokens, ff, ld);
+    else
+        hipLaunchKernelGGL((gelu_gate_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, y, gu, tokens, ff, ld);
+    return launched("stack_gelu_gate");
+}
+
+static bool attn_shape_ok(const StackAttnParams& p, const char* what)
+{
+    if (!known_dtype(p.dtype, what))
+        return false;
+    if (p.heads < 1 || p.kv_heads < 1 || p.heads % p.kv_heads || p.maps < 1 || p.maps > 2 || p.dim < 1 || p.vdim < 1 || p.page < 1
+        || p.max_blocks < 1)
+    {
+        set_error("%s: heads %d, kv_heads %d, maps %d, dim %d, vdim %d, page %d, max_blocks %d is not a shape it serves", what, p.heads,
+            p.kv_heads, p.maps, p.dim, p.vdim, p.page, p.max_blocks);
+        return false;
+    }
+    if ((p.dim & 1) || (p.rot_dims & 1) || p.rot_dims > p.dim || p.rot_dims < 0)
+    {
+        set_error("%s: the rotation pairs neighbours: dim %d and rot_dims %d must be even, rot_dims <= dim", what, p.dim, p.rot_dims);
+        return false;
+    }
+    return true;
+}
+
+int launch_stack_rope_kv(const StackAttnParams& p, hipStream_t stream)
+{
+    if (p.tokens <= 0)
+        return 0;
+    if (!attn_shape_ok(p, "stack_rope_kv"))
+        return -1;
+    if (p.dtype == DT_BF16)
+        hipLaunchKernelGGL((rope_kv_kernel<DT_BF16>), dim3(p.tokens), dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL((rope_kv_kernel<DT_FLOAT>), dim3(p.tokens), dim3(256), 0, stream, p);
+    return launched("stack_rope_kv");
+}
+
+int launch_stack_attention_general(const StackAttnParams& p, hipStream_t stream)
+{
+    // (the dispatcher launch_stack_attention lives in stack_attn.hip)
+    if (p.tokens <= 0)
+        return 0;
+    if (!attn_shape_ok(p, "stack_attention"))
+        return -1;
+    if (p.vdim > AT * A_CPT)
+    {
+        set_error("stack_attention: vdim %d is beyond the %d channels the general kernel keeps", p.vdim, AT * A_CPT);
+        return -1;
+    }
+    const size_t lds = sizeof(float) * ((size_t) p.maps * p.dim + (size_t) p.maps * AT + 32);
+    const dim3 grid(p.tokens, p.heads);
+#define TLLM_ATTN_GEN(DT, MAPS) hipLaunchKernelGGL((attn_general_kernel<DT, MAPS>), grid, dim3(AT), lds, stream, p)
+    if (p.dtype == DT_BF16)
+    {
+        if (p.maps == 2)
+            TLLM_ATTN_GEN(DT_BF16, 2);
+        else
+            TLLM_ATTN_GEN(DT_BF16, 1);
+    }
+    else
+    {
+        if (p.maps == 2)
+            TLLM_ATTN_GEN(DT_FLOAT, 2);
+        else
+            TLLM_ATTN_GEN(DT_FLOAT, 1);
+    }
+#undef TLLM_ATTN_GEN
+    return launched("stack_attention");
+}
+
+float stack_rope_freqs(float* freq, int32_t dims, double base, double factor, double original, double fast, double slow)
+{
+    const int n = dims / 2;
+    const double two_pi = 6.283185307179586476925286766559;
+    double lo = 0, hi = 0;
+    if (factor > 0)
+    {
+        auto dim_of = [&](double turns) { return dims * std::log(original / (two_pi * turns)) / (2.0 * std::log(base)); };
+        lo = std::max(std::floor(dim_of(fast)), 0.0);
+        hi = std::min(std::ceil(dim_of(slow)), (double) (dims - 1));
+    }
+    for (int i = 0; i < n; ++i)
+    {
+        double f = std::pow(base, -2.0 * i / dims);
+        if (factor > 0)
+        {
+            double ramp = (i - lo) / std::max(hi - lo, 0.001);
+            ramp = ramp < 0 ? 0 : (ramp > 1 ? 1 : ramp);
+            f = f / factor * ramp + f * (1 - ramp);
+        }
+        freq[i] = (float) f;
+    }
+    return factor > 0 ? (float) (0.1 * std::log(factor) + 1.0) : 1.f;
+}
+
+int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
+{
+    if (p.tokens <= 0 || p.entries <= 0)
+        return 0;
+    if (!known_dtype(p.dtype, "stack_hgrn2"))
+        return -1;
+    if (p.heads < 1 || p.dim < 1 || p.vdim < 1 || p.dim > 128)
+    {
+        set_error("stack_hgrn2: heads %d, dim %d, vdim %d is not a shape it serves (dim <= 128: a state column lives in registers)", p.heads,
+            p.dim, p.vdim);
+        return -1;
+    }
+    const dim3 grid(p.entries, p.heads, (p.vdim + 63) / 64);
+#define TLLM_HGRN(DT, DMAX) hipLaunchKernelGGL((hgrn2_scan_kernel<DT, DMAX>), grid, dim3(64), 0, stream, p)
+#define TLLM_HGRN_D(DT)                                                                                                         \
+    do                                                                                                                              \
+    {                                                                                                                               \
+        if (p.dim <= 16)                                                                                                            \
+            TLLM_HGRN(DT, 16);                                                                                                      \
+        else if (p.dim <= 32)                                                                                                       \
+            TLLM_HGRN(DT, 32);                                                                                                      \
+        else if (p.dim <= 64)                                                                                                       \
+            TLLM_HGRN(DT, 64);                                                                                                      \
+        else                                                                                                                        \
+            TLLM_HGRN(DT, 128);                                                                                                     \
+    } while (0)
+    if (p.dtype == DT_BF16)
+        TLLM_HGRN_D(DT_BF16);
+    else
+        TLLM_HGRN_D(DT_FLOAT);
+#undef TLLM_HGRN_D
+#undef TLLM_HGRN
+    if (launched("stack_hgrn2 scan"))
+        return -1;
+    const int64_t nh = (int64_t) p.tokens * p.heads;
+    if (p.dtype == DT_BF16)
+        hipLaunchKernelGGL((head_rmsnorm_kernel<DT_BF16>), dim3((unsigned) ((nh + 3) / 4)), dim3(256), 0, stream, p.out, p.o32, p.norm_w, nh,
+            p.vdim, p.eps);
+    else
+        hipLaunchKernelGGL((head_rmsnorm_kernel<DT_FLOAT>), dim3((unsigned) ((nh + 3) / 4)), dim3(256), 0, stream, p.out, p.o32, p.norm_w, nh,
+            p.vdim, p.eps);
+    return launched("stack_hgrn2 norm");
+}
+
+} // namespace kernels
+} // namespace tllm

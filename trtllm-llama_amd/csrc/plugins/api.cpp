@@ -7,26 +7,6 @@
 #include <cstdio>
 #include <mutex>
 
-namespace tllm
-{
-
-static thread_local char g_err[2048] = {0};
-
-void set_error(const char* fmt, ...)
-{
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_err, sizeof(g_err), fmt, ap);
-    va_end(ap);
-}
-
-const char* last_error()
-{
-    return g_err;
-}
-
-} // namespace tllm
-
 using namespace tllm;
 using namespace tllm::plugins;
 
@@ -122,11 +102,6 @@ bool initLibNvInferPlugins(void* logger, const char* libNamespace)
 int32_t getInferLibVersion(void)
 {
     return 103; // 0.1.3, the vendored tensorrt_llm package version (T/setup.py:22)
-}
-
-const char* tllm_last_error(void)
-{
-    return last_error();
 }
 
 int32_t tllm_plugin_registry_size(void)

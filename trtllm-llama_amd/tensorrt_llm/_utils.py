@@ -83,3 +83,29 @@ def mpi_world_size():
         if k in os.environ:
             return int(os.environ[k])
     return 1
+
+
+def read_safetensors(path):
+    """name -> (numpy array, kind) from a safetensors file (8-byte little-endian header length, JSON header, raw data), without
+    executing anything from it.  bfloat16 tensors come back as their uint16 bit patterns with kind 'bfloat16' (numpy has no such
+    type); F32 / F16 / I32 / I64 as themselves with kind = the numpy dtype's name."""
+    import json
+    import struct
+    kinds = {'BF16': (np.uint16, 'bfloat16'), 'F32': (np.float32, 'float32'), 'F16': (np.float16, 'float16'),
+             'I32': (np.int32, 'int32'), 'I64': (np.int64, 'int64')}
+    with open(path, 'rb') as f:
+        (n, ) = struct.unpack('<Q', f.read(8))
+        header = json.loads(f.read(n))
+        base = 8 + n
+        out = {}
+        for name, meta in header.items():
+            if name == '__metadata__':
+                continue
+            if meta['dtype'] not in kinds:
+                raise ValueError(f"{path}: tensor {name} has dtype {meta['dtype']}, which this reader does not take")
+            np_dt, kind = kinds[meta['dtype']]
+            lo, hi = meta['data_offsets']
+            f.seek(base + lo)
+            a = np.frombuffer(f.read(hi - lo), np_dt).reshape(meta['shape'])
+            out[name] = (a, kind)
+    return out

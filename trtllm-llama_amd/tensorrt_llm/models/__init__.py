@@ -1,4 +1,7 @@
 from .llama.model import LLaMADecoderLayer, LLaMAForCausalLM, LLaMAModel
 from .quantized.quant import smooth_quantize, weight_only_quantize
+from .registry import MODEL_REGISTRY, load_model, model_class_for
+from .tolenex.model import TolenexConfig, TolenexForCausalLM
 
-__all__ = ['LLaMADecoderLayer', 'LLaMAForCausalLM', 'LLaMAModel', 'smooth_quantize', 'weight_only_quantize']
+__all__ = ['LLaMADecoderLayer', 'LLaMAForCausalLM', 'LLaMAModel', 'smooth_quantize', 'weight_only_quantize', 'MODEL_REGISTRY',
+           'load_model', 'model_class_for', 'TolenexConfig', 'TolenexForCausalLM']

@@ -1,6 +1,7 @@
-from .generation import GenerationSession, ModelConfig, SamplingConfig
-from .kv_cache_manager import GenerationSequence, KVCacheManager
+from .generation import GenerationSession, ModelConfig, RaggedGenerationSession, SamplingConfig
+from .kv_cache_manager import GenerationSequence, KVCacheManager, StateSlotManager
+from .scheduler import RaggedScheduler, Request
 from .session import Session, TensorInfo
 
-__all__ = ['ModelConfig', 'GenerationSession', 'GenerationSequence', 'KVCacheManager', 'SamplingConfig', 'Session',
+__all__ = ['ModelConfig', 'GenerationSession', 'RaggedGenerationSession', 'RaggedScheduler', 'Request', 'StateSlotManager', 'GenerationSequence', 'KVCacheManager', 'SamplingConfig', 'Session',
            'TensorInfo']

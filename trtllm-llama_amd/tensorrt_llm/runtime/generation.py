@@ -144,3 +144,138 @@ class GenerationSession(object):
         for i, x in enumerate(input_ids):
             padded[i, :lens[i]] = np.asarray(x.cpu() if hasattr(x, 'cpu') else x)
         return self.decode(padded, lens, sampling_config)
+
+
+class RaggedGenerationSession(object):
+    """Generation over the ragged stack engine (runtime/stack.py): the counterpart of GenerationSession for models that are
+    served in packed steps - portions of prompts beside single decoded tokens - with a paged cache and per-sequence state slots.
+
+        session = RaggedGenerationSession(model, dtype='bfloat16', max_tokens=4096, max_sequences=4)
+        outputs = session.decode_batch(prompts, SamplingConfig(end_id=.., pad_id=..), max_new_tokens=32)
+
+    decode_batch lets the scheduler (RaggedScheduler) compose the steps; `step` runs one step the caller composed (a replay of a
+    recorded schedule, a test of a particular cut).  Both go through the same cache managers and the same engine step.
+    `model` is a model object of the registry (tensorrt_llm.models) that can describe itself to the engine."""
+
+    def __init__(self, model, dtype: str = 'bfloat16', max_tokens: int = 4096, max_sequences: int = 4, max_batch_tokens: int = 2048,
+                 debug_mode: bool = False, build_if_missing: bool = False):
+        from .kv_cache_manager import GenerationSequence, KVCacheManager, StateSlotManager
+        self._Sequence = GenerationSequence
+        self.model = model
+        page = model.page_size
+        blocks = -(-max_tokens // page)
+        self.engine = model.build_stack_engine(dtype=dtype, num_blocks=blocks, num_slots=max_sequences, debug_taps=debug_mode,
+                                               build_if_missing=build_if_missing)
+        self.page_size, self.num_blocks, self.max_sequences = page, blocks, max_sequences
+        self.max_batch_tokens = max_batch_tokens
+        self.cache = KVCacheManager(None, blocks, page, max_blocks_per_seq=blocks)
+        self.slots = StateSlotManager(max_sequences)
+        self._seq = {}   # request id -> GenerationSequence
+        self._len = {}   # request id -> tokens it holds
+        self._next_seq_idx = 0
+
+    @property
+    def vocab_size(self):
+        return self.engine.vocab
+
+    def live(self):
+        return list(self._seq)
+
+    def length_of(self, rid) -> int:
+        return self._len[rid]
+
+    def step(self, entries, end=(), return_logits: bool = True):
+        """entries: [(request id, tokens, want)] - the next tokens of each request and the places among them whose logits /
+        next-token choice are asked for.  A request is admitted at its first entry (slot + blocks), `end` lists the requests
+        that give back what they hold after this step.  Returns (logits fp32 [wanted, vocab] or None, next ids int32 [wanted]),
+        rows in the order of the entries and of their `want`."""
+        tokens, counts, pos0, slots, want_rows, seqs = [], [], [], [], [], []
+        seen = set()
+        for rid, toks, want in entries:
+            toks = [int(t) for t in toks]
+            if not toks:
+                raise ValueError(f'request {rid}: an entry without tokens')
+            if rid in seen:
+                raise ValueError(f'request {rid} appears twice in one step')
+            seen.add(rid)
+            if rid not in self._seq:
+                self._seq[rid] = self._Sequence(self._next_seq_idx, len(self._seq))
+                self._next_seq_idx += 1
+                self._len[rid] = 0
+            seq = self._seq[rid]
+            slot = self.slots.acquire(seq)
+            self.cache.reserve(seq, self._len[rid] + len(toks))
+            for w in want:
+                if not 0 <= int(w) < len(toks):
+                    raise ValueError(f'request {rid}: wanted place {w} is outside its {len(toks)} tokens')
+                want_rows.append(len(tokens) + int(w))
+            tokens += toks
+            counts.append(len(toks))
+            pos0.append(self._len[rid])
+            slots.append(slot)
+            seqs.append(seq)
+        out = (None, np.empty(0, np.int32))
+        if entries:
+            max_blocks = max(-(-(p + c) // self.page_size) for p, c in zip(pos0, counts))
+            table = self.cache.blocks_manager.block_table(seqs, max_blocks)
+            out = self.engine.step(tokens, counts, pos0, slots, table, want_rows, return_logits=return_logits)
+            for (rid, toks, _) in entries:
+                self._len[rid] += len(toks)
+        for rid in end:
+            self.release(rid)
+        return out
+
+    def release(self, rid):
+        seq = self._seq.pop(rid, None)
+        if seq is None:
+            return
+        self.cache.release(seq)
+        self.slots.release(seq)
+        del self._len[rid]
+
+    def decode_batch(self, prompts, sampling_config: SamplingConfig, max_new_tokens: int):
+        """Greedy generation for a list of prompts of any lengths through the scheduler: more prompts than state slots queue up,
+        long prompts are cut into portions by the step's token budget.  Returns a list of int32 arrays (the generated tokens,
+        up to and including end_id)."""
+        from .scheduler import RaggedScheduler, Request
+        GenerationSession._check_sampling_config(sampling_config)
+        if sampling_config.num_beams != 1:
+            raise NotImplementedError('beam search is not built for the ragged engine: greedy only')
+        sched = RaggedScheduler(self.max_batch_tokens, self.max_sequences, self.page_size, self.num_blocks)
+        base = ('decode_batch', id(sched))
+        reqs = [Request((base, i), [int(t) for t in (p.tolist() if hasattr(p, 'tolist') else p)], max_new_tokens,
+                        sampling_config.end_id) for i, p in enumerate(prompts)]
+        for r in reqs:
+            sched.add(r)
+        while sched.has_work():
+            plan = sched.schedule()
+            if not plan:
+                raise RuntimeError('the scheduler has work but cannot place any of it (pool too small for the next request)')
+            entries, asks = [], []
+            for r, n in plan:
+                toks = r.tokens()[r.fed:r.fed + n]
+                last = r.fed + n == len(r.prompt) + len(r.output)
+                entries.append((r.rid, toks, [n - 1] if last else []))
+                asks.append(last)
+            _, ids = self.step(entries, return_logits=False)
+            k = 0
+            for (r, n), last in zip(plan, asks):
+                nid = None
+                if last:
+                    nid = int(ids[k])
+                    k += 1
+                if sched.update(r, n, nid):
+                    self.release(r.rid)
+        return [np.asarray(r.output, np.int32) for r in reqs]
+
+    def decode(self, input_ids, input_lengths, sampling_config: SamplingConfig, max_new_tokens: int):
+        """GenerationSession.decode's shape: int32 [batch, max_input_length] padded ids + lengths in, int32
+        [batch, 1, max_input_length + max_new_tokens] out (prompt, generated tokens, pad_id behind them)."""
+        ids = input_ids.cpu().numpy() if hasattr(input_ids, 'cpu') else np.asarray(input_ids)
+        lens = input_lengths.cpu().numpy() if hasattr(input_lengths, 'cpu') else np.asarray(input_lengths)
+        outs = self.decode_batch([ids[b, :lens[b]] for b in range(ids.shape[0])], sampling_config, max_new_tokens)
+        full = np.full((ids.shape[0], 1, ids.shape[1] + max_new_tokens), sampling_config.pad_id, np.int32)
+        for b, o in enumerate(outs):
+            full[b, 0, :lens[b]] = ids[b, :lens[b]]
+            full[b, 0, ids.shape[1]:ids.shape[1] + len(o)] = o
+        return full

@@ -6,7 +6,11 @@ kv_cache_manager.py:84-96).  The manager hands block ids to sequences; the GPTAt
 see the resulting table of device pointers [sequences, beam_width, 2, max_blocks_per_seq] (int64, shipped as int32 pairs:
 gptAttentionPlugin.cpp:313-325, K/kvCacheUtils.h:34-112).
 
-Pools are torch tensors (data_ptr / element_size / numel) or anything with the same three members.
+Pools are torch tensors (data_ptr / element_size / numel) or anything with the same three members.  An engine that owns its
+pools and addresses blocks by id (the ragged stack engine: one id is valid in every layer's pool) passes no pools at all and
+reads `block_ids` / `block_table` instead of pointers.
+
+`StateSlotManager` is the same idea for recurrent layers: a fixed number of per-sequence state slots, handed out and taken back.
 """
 import collections
 from typing import List
@@ -48,7 +52,7 @@ class BlocksManager(object):
     def __init__(self, memory_pools: List, blocks: int, max_blocks_per_seq: int = 128, beam_width: int = 1):
         self.memory_pools, self.blocks = memory_pools, blocks
         self.max_blocks_per_seq, self.beam_width = max_blocks_per_seq, beam_width
-        self._geom = [_pool_geometry(p, blocks) for p in memory_pools]
+        self._geom = [_pool_geometry(p, blocks) for p in (memory_pools or [])]
         self._refs = np.zeros(blocks, np.int64)
         self._free = collections.deque(range(blocks))
         self._owned = {}  # owner -> [beam][logical block] -> block id
@@ -98,6 +102,14 @@ class BlocksManager(object):
                 if self._refs[blk] == 0:
                     self._free.append(blk)
 
+    def block_table(self, owners: List[GenerationSequence], max_blocks: int):
+        """int32 [len(owners), max_blocks] of block ids (beam 0), zero-padded: what an engine that addresses blocks by id takes."""
+        table = np.zeros((len(owners), max_blocks), np.int32)
+        for i, owner in enumerate(owners):
+            ids = self._owned.get(owner, [[]])[0]
+            table[i, :len(ids)] = ids
+        return table
+
     # -- what the kernels consume
     def get_pointer_array(self, pool_idx: int):
         """int64 [sequences, beam_width, 2, max_blocks_per_seq] (numpy): K and V block addresses, 0 where unallocated."""
@@ -120,7 +132,7 @@ class KVCacheManager(object):
         if tokens_per_block < 1 or tokens_per_block & (tokens_per_block - 1):
             raise ValueError('tokens_per_block must be a power of two')
         self.blocks_manager = BlocksManager(memory_pools, blocks, max_blocks_per_seq, beam_width)
-        self.num_pools, self.tokens_per_block, self.beam_width = len(memory_pools), tokens_per_block, beam_width
+        self.num_pools, self.tokens_per_block, self.beam_width = len(memory_pools or []), tokens_per_block, beam_width
         self.lens, self.sequences = [], []
 
     def add_sequence(self, sequence: GenerationSequence, context_len: int):
@@ -132,6 +144,31 @@ class KVCacheManager(object):
         self.lens.append(context_len)
         for _ in range(-(-(context_len + 1) // self.tokens_per_block)):
             self.blocks_manager.allocate(sequence, share_across_beam=True)
+
+    def reserve(self, sequence: GenerationSequence, total_tokens: int):
+        """Ragged batches: make `sequence` (known or new) hold blocks for `total_tokens` tokens.  A prompt arrives in portions of
+        any size, so the blocks are taken as the portions come, not for the whole prompt at once."""
+        if sequence not in self.blocks_manager._owned and sequence not in self.sequences:
+            sequence.batch_idx = len(self.sequences)
+            self.sequences.append(sequence)
+            self.lens.append(0)
+        have = self.blocks_manager.get_number_blocks(sequence) if sequence in self.blocks_manager._owned else 0
+        need = -(-total_tokens // self.tokens_per_block)
+        if need - have > self.blocks_manager.num_free_blocks():
+            raise RuntimeError(f"Can't allocate new block for KV cache: sequence {sequence.get_seq_idx()} needs {need - have} more, "
+                               f'{self.blocks_manager.num_free_blocks()} are free')
+        for _ in range(need - have):
+            self.blocks_manager.allocate(sequence, share_across_beam=True)
+        self.lens[self.sequences.index(sequence)] = total_tokens
+
+    def release(self, sequence: GenerationSequence):
+        """Give back everything `sequence` holds (ragged batches: a sequence ends when its owner says so)."""
+        i = self.sequences.index(sequence)
+        if sequence in self.blocks_manager._owned:
+            self.blocks_manager.free(sequence)
+        del self.sequences[i], self.lens[i]
+        for j, seq in enumerate(self.sequences):
+            seq.batch_idx = j
 
     def step(self, finished: List[bool]):
         keep_seq, keep_len = [], []
@@ -155,3 +192,34 @@ class KVCacheManager(object):
             t = torch.from_numpy(self.blocks_manager.get_pointer_array(pool))
             out.append((t.to(device) if device else t).view(dtype=torch.int32))
         return out
+
+
+class StateSlotManager(object):
+    """Per-sequence state slots of recurrent layers: `slots` of them, the lowest free one first, so a slot that was given back is
+    the next one used.  The engine zeroes nothing on release: a sequence that starts at position 0 starts from a zero state."""
+
+    def __init__(self, slots: int):
+        if slots < 1:
+            raise ValueError('at least one state slot')
+        self.slots = slots
+        self._free = list(range(slots))
+        self._owner = {}
+
+    def num_free_slots(self) -> int:
+        return len(self._free)
+
+    def acquire(self, sequence: GenerationSequence) -> int:
+        if sequence in self._owner:
+            return self._owner[sequence]
+        if not self._free:
+            raise RuntimeError(f'all {self.slots} state slots are in use')
+        slot = min(self._free)
+        self._free.remove(slot)
+        self._owner[sequence] = slot
+        return slot
+
+    def slot_of(self, sequence: GenerationSequence) -> int:
+        return self._owner[sequence]
+
+    def release(self, sequence: GenerationSequence):
+        self._free.append(self._owner.pop(sequence))
