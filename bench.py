@@ -21,6 +21,8 @@ import os
 import sys
 import time
 
+import numpy as np
+
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, 'trtllm-llama_amd'))
 sys.path.insert(0, ROOT)
@@ -60,6 +62,11 @@ def parse():
     ap.add_argument('--parity-prompts', type=int, default=8, help='seeded prompts of the accuracy report')
     ap.add_argument('--cpu-tokens', type=int, default=0, help='CPU-baseline decode steps (0 = sized to ~20 s)')
     ap.add_argument('--cpu-threads', type=int, default=0)
+    ap.add_argument('--design', default='llama', choices=['llama', 'tolenex'],
+                    help="tolenex: a side report instead of the headline workload - prefill and decode throughput of the Tolenex design "
+                         "(bfloat16, ragged stack engine) at layer sizes of real models, beside LLaMA fp16 at equal size")
+    ap.add_argument('--design-sizes', default='2048,4096', help='--design tolenex: comma list of model widths')
+    ap.add_argument('--design-layers', type=int, default=4, help='--design tolenex: layers of both models')
     ap.add_argument('--cpu-sweep', default='', help='debug: comma list of thread counts to try (stderr)')
     return ap.parse_args()
 
@@ -568,6 +575,97 @@ def cpu_baseline(n_tokens, context, threads=0, sweep=None, model=None, layers=32
                         f'{dt:.1f} s timed, {build_s:.0f} s untimed set-up'))
 
 
+def tolenex_config(width, layers, vocab=32000):
+    """A Tolenex configuration with the layer sizes of a LLaMA-like model of this width: attention heads of 2 x 64 query / key
+    dimensions (two maps) and 128 value dimensions, four query heads per key / value head, every fourth layer an HGRN2 layer with
+    128 x 128 states, feed-forward 2.6875 x width."""
+    heads = width // 128
+    attn = {'type': 'attention', 'mlp': {'ff': int(width * 2.6875), 'kind': 'dense'},
+            'mixer': {'heads': heads, 'kv_heads': max(heads // 4, 1), 'dim': 64, 'vdim': 128, 'diff': 0.3, 'scale': 0.125, 'softcap': 50.0,
+                      'rot': {'dims': 64, 'base': 1000000.0, 'scaling': {'factor': 8.0, 'original': 4096, 'fast': 32.0, 'slow': 1.0}}}}
+    rec = {'type': 'hgrn2', 'mlp': {'ff': int(width * 2.6875), 'kind': 'dense'}, 'mixer': {'heads': heads, 'dim': 128, 'vdim': 128}}
+    return {'architecture': 'Tolenex', 'vocab': vocab, 'width': width, 'embedding': {'scale': 8.0}, 'norm': {'eps': 1e-5, 'groups': 2},
+            'layers': [rec if i % 4 == 2 else attn for i in range(layers)]}
+
+
+def tolenex_report(torch, args, dev):
+    """Prefill (one step of S prompt tokens) and decode (single tokens at context S, 1 and 4 sequences per step) of Tolenex in
+    bfloat16 through RaggedGenerationSession.step, and the same two phases of LLaMA fp16 (the closest model the framework has: same
+    width, layers, heads x 128, feed-forward size, vocabulary; unquantised) through NativeSession.  Random weights; wall clock around
+    synchronised calls, nothing else in the timed regions."""
+    from tensorrt_llm.models import TolenexForCausalLM
+    from tensorrt_llm.runtime import RaggedGenerationSession
+    from tensorrt_llm.runtime.native import NativeSession
+    S, K, W = args.context, min(args.steps, 64), max(min(args.warmup, 8), 2)
+    rows = []
+    for width in [int(v) for v in args.design_sizes.split(',')]:
+        L = args.design_layers
+        cfg = tolenex_config(width, L)
+        model = TolenexForCausalLM.from_random(cfg, seed=1)
+        sess = RaggedGenerationSession(model, dtype='bfloat16', max_tokens=4 * (S + 2 * K + 2 * W + 64), max_sequences=4,
+                                       max_batch_tokens=S)
+        rng = np.random.default_rng(0)
+        prompt = rng.integers(0, cfg['vocab'], S).tolist()
+        row = dict(width=width, layers=L, context=S, weight_bytes=sess.engine.weight_bytes())
+        sess.step([('warm', prompt, [S - 1])], end=['warm'])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        sess.step([('p', prompt, [S - 1])])
+        t_prefill = time.perf_counter() - t0
+        row['tolenex_prefill_ms'] = t_prefill * 1e3
+        row['tolenex_prefill_tokens_per_s'] = S / t_prefill
+        for batch in (1, 4):
+            ids = ['p'] + [f'q{b}' for b in range(1, batch)]
+            for rid in ids[1:]:
+                sess.step([(rid, prompt, [])])
+            for _ in range(W):
+                sess.step([(rid, [7], [0]) for rid in ids], return_logits=False)
+            t0 = time.perf_counter()
+            for _ in range(K):
+                sess.step([(rid, [7], [0]) for rid in ids], return_logits=False)
+            dt = time.perf_counter() - t0
+            row[f'tolenex_decode_b{batch}_tokens_per_s'] = batch * K / dt
+            row[f'tolenex_decode_b{batch}_ms_per_step'] = dt * 1e3 / K
+            ctx = sess.length_of('p')
+            row[f'tolenex_decode_b{batch}_hbm_fraction'] = sess.engine.step_bytes(batch, batch * ctx, batch) / (dt / K) / 8e12
+        del sess, model
+        # LLaMA fp16 at equal size
+        lc = dict(num_layers=L, num_heads=width // 128, hidden_size=width, inter_size=int(width * 2.6875), vocab_size=cfg['vocab'],
+                  max_position_embeddings=S + 2 * K + 2 * W + 64, rms_norm_eps=1e-5, quant_mode=0)
+        ls = NativeSession(lc)
+        for k, v in synth_weights(torch, lc, 'fp16', False, 1, 0, dev).items():
+            ls.set_tensor(k, v)
+        ls.finalize()
+        stream = torch.cuda.current_stream().cuda_stream
+        ids = np.asarray([prompt], np.int32)
+        lens = np.asarray([S], np.int32)
+        for batch in (1, 4):
+            ls.setup(batch, S, 2 * K + 2 * W + 8)
+            bi, bl = np.repeat(ids, batch, 0), np.repeat(lens, batch, 0)
+            ls.context(bi, bl, stream)
+            torch.cuda.synchronize()
+            if batch == 1:
+                t0 = time.perf_counter()
+                ls.context(bi, bl, stream)
+                torch.cuda.synchronize()
+                row['llama_prefill_ms'] = (time.perf_counter() - t0) * 1e3
+                row['llama_prefill_tokens_per_s'] = S / (time.perf_counter() - t0)
+            ls.step(2, use_graph=False, stream=stream)
+            ls.step(W, use_graph=True, stream=stream)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ls.step(K, use_graph=True, stream=stream)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            row[f'llama_decode_b{batch}_tokens_per_s'] = batch * K / dt
+            row[f'llama_decode_b{batch}_ms_per_step'] = dt * 1e3 / K
+        ls.close()
+        rows.append({k: (round(v, 3) if isinstance(v, float) else v) for k, v in row.items()})
+        print(f'[bench] {rows[-1]}', file=sys.stderr, flush=True)
+    print(json.dumps({'metric': 'tolenex_side_report', 'dtype': 'bf16 (Tolenex) / fp16 (LLaMA)', 'data': 'synthetic', 'n_gpus': 1,
+                      'steps': K, 'warmup': W, 'sizes': rows}))
+
+
 def main():
     args = parse()
     import torch
@@ -598,6 +696,10 @@ def main():
         local = 0
     torch.cuda.set_device(local)
     dev = torch.device('cuda', local)
+    if args.design == 'tolenex':
+        if world != 1:
+            raise SystemExit('--design tolenex is a one-GPU report')
+        return tolenex_report(torch, args, dev)
     dist = None
     if world > 1:
         import torch.distributed as dist

@@ -37,6 +37,11 @@ def check(got, want, tol, what=''):
 FULL = [attention_layer(), hgrn2_layer(ff=72), attention_layer(heads=4, kv_heads=4, dim=24, vdim=16, rot_dims=24, ff=0),
         hgrn2_layer(heads=3, dim=16, vdim=32, ff=40), attention_layer(kv_heads=1, rot_dims=0, softcap=0.0)]
 
+# shapes the MFMA tile kernel takes in bfloat16 (dim and vdim of 32 / 64 / 128); fp32 runs them on the general kernel
+TILED = [attention_layer(heads=6, kv_heads=2, dim=32, vdim=32, rot_dims=16), hgrn2_layer(heads=2, dim=32, vdim=64, ff=72),
+         attention_layer(heads=2, kv_heads=1, dim=64, vdim=128, rot_dims=64, ff=0), attention_layer(heads=3, kv_heads=3, dim=32, vdim=64, rot_dims=0)]
+STACKS = {'general': FULL, 'tiled': TILED}
+
 MECHANISMS = {
     'attention_alone_no_ff': make_config([attention_layer(ff=0)]),
     'attention_one_group': make_config([attention_layer()], groups=1),
@@ -44,6 +49,10 @@ MECHANISMS = {
     'attention_no_rotation_no_cap': make_config([attention_layer(rot_dims=0, softcap=0.0)]),
     'attention_every_head_its_own_kv': make_config([attention_layer(heads=4, kv_heads=4)]),
     'attention_one_kv_head_odd_sizes': make_config([attention_layer(heads=5, kv_heads=1, dim=12, vdim=20, rot_dims=4)], width=80, groups=5),
+    'attention_tile_32_32': make_config([TILED[0]]),
+    'attention_tile_64_128': make_config([TILED[2]]),
+    'attention_tile_128_64_one_map_group': make_config([attention_layer(heads=2, kv_heads=2, dim=128, vdim=64, rot_dims=32, softcap=0.0)]),
+    'tiled_stack_looped': make_config(TILED, loop=(1, 3, 2), groups=2),
     'attention_wide_values': make_config([attention_layer(heads=2, kv_heads=1, dim=8, vdim=160)]),
     'hgrn2_alone_no_ff': make_config([hgrn2_layer()]),
     'hgrn2_small_heads': make_config([hgrn2_layer(heads=4, dim=8, vdim=8, ff=48)], groups=2),
@@ -81,9 +90,10 @@ def test_residual_stream_behind_every_layer_run():
         assert np.abs(s.engine.tap(j) - x).max() < 2e-4 * np.abs(x).max(), f'layer run {j}'
 
 
+@pytest.mark.parametrize('stack', sorted(STACKS))
 @pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
-def test_prefill_then_token_by_token(dtype):
-    cfg = MECHANISMS['loop_in_the_middle']
+def test_prefill_then_token_by_token(dtype, stack):
+    cfg = make_config(STACKS[stack], loop=(1, 4, 2), groups=4)
     w = random_weights(cfg, seed=5)
     toks = tokens_for(cfg, 150, 3)
     want = O.tolenex_logits(toks, as_f64(w), cfg)
@@ -94,8 +104,9 @@ def test_prefill_then_token_by_token(dtype):
 
 @pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
 @pytest.mark.parametrize('sizes', [[2] * 40, [3, 61, 2, 64, 1, 5, 2, 58, 1, 1, 2], [63, 2, 63, 1, 1, 66], [1] * 9 + [120, 2]])
-def test_portions_of_a_prompt(sizes, dtype):
-    cfg = make_config(FULL, loop=(0, 4, 2))
+@pytest.mark.parametrize('stack', sorted(STACKS))
+def test_portions_of_a_prompt(sizes, dtype, stack):
+    cfg = make_config(STACKS[stack], loop=(0, 4, 2))
     w = random_weights(cfg, seed=7)
     toks = tokens_for(cfg, sum(sizes), 4)
     want = O.tolenex_logits(toks, as_f64(w), cfg)
@@ -105,8 +116,9 @@ def test_portions_of_a_prompt(sizes, dtype):
 
 
 @pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
-def test_unequal_requests_in_one_batch_equal_each_alone(dtype):
-    cfg = make_config(FULL, loop=(1, 3, 2))
+@pytest.mark.parametrize('stack', sorted(STACKS))
+def test_unequal_requests_in_one_batch_equal_each_alone(dtype, stack):
+    cfg = make_config(STACKS[stack], loop=(1, 3, 2))
     w = random_weights(cfg, seed=9)
     reqs = {'a': tokens_for(cfg, 131, 5), 'b': tokens_for(cfg, 9, 6), 'c': tokens_for(cfg, 66, 7), 'd': tokens_for(cfg, 2, 8)}
     schedule = [[('a', 60), ('b', 2)], [('b', 1), ('a', 5), ('c', 64)], [('c', 1), ('b', 1), ('a', 1), ('d', 2)],
@@ -165,11 +177,11 @@ def test_pool_exhaustion_is_an_error_not_a_fault():
         s.step([('d', [1], [0])])
 
 
-def _far_key_case(p_far, n, seed):
+def _far_key_case(p_far, n, seed, D=16):
     """One attention layer whose head 0, map 0 is rigged so that the LAST token's query meets the key of the token at p_far with
     a score far above all others (a bump on a dimension the rotation leaves alone): dropping, shifting or corrupting that one
     far key changes the logits at the last position by much more than bfloat16 rounding."""
-    cfg = make_config([attention_layer(heads=2, kv_heads=1, dim=16, vdim=24, rot_dims=8, ff=0, softcap=60.0)], groups=2)
+    cfg = make_config([attention_layer(heads=2, kv_heads=1, dim=D, vdim=24 if D == 16 else 64, rot_dims=8, ff=0, softcap=60.0)], groups=2)
     w = random_weights(cfg, seed=seed)
     rng = np.random.default_rng(seed)
     far_tok, last_tok = 3, 4
@@ -178,18 +190,17 @@ def _far_key_case(p_far, n, seed):
     wf = as_f64(w)
     h = O.grouped_rms_norm(wf['embed'] * cfg['embedding']['scale'], wf['l0.norm1'], cfg['norm']['groups'], cfg['norm']['eps'])
     alpha = (30.0 / cfg['layers'][0]['mixer']['scale']) ** 0.5
-    D = 16
     from tolenex_cases import bf16_round
-    w['l0.mix.q'][0 * D + 15] = bf16_round((alpha * h[last_tok] / (h[last_tok] @ h[last_tok])).astype(np.float32))
-    w['l0.mix.k'][0 * D + 15] = bf16_round((alpha * h[far_tok] / (h[far_tok] @ h[far_tok])).astype(np.float32))
+    w['l0.mix.q'][0 * D + D - 1] = bf16_round((alpha * h[last_tok] / (h[last_tok] @ h[last_tok])).astype(np.float32))
+    w['l0.mix.k'][0 * D + D - 1] = bf16_round((alpha * h[far_tok] / (h[far_tok] @ h[far_tok])).astype(np.float32))
     return cfg, w, toks
 
 
-@pytest.mark.parametrize('p_far', [0, 1, 63, 64, 127, 128, 200])
-@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
-def test_a_far_key_that_decides_the_answer(p_far, dtype):
+@pytest.mark.parametrize('p_far', [0, 1, 31, 32, 63, 64, 127, 128, 200])
+@pytest.mark.parametrize('dtype,D', [('float32', 16), ('bfloat16', 16), ('bfloat16', 32)])
+def test_a_far_key_that_decides_the_answer(p_far, dtype, D):
     n = 333
-    cfg, w, toks = _far_key_case(p_far, n, seed=40 + p_far)
+    cfg, w, toks = _far_key_case(p_far, n, seed=40 + p_far, D=D)
     wf = as_f64(w)
     want = O.tolenex_logits(toks, wf, cfg)
     other = list(toks)
@@ -214,8 +225,9 @@ def test_first_tokens_of_a_sequence():
         check(replay(s, {-n: toks}, [[(-n, 1)]] * n)[-n], O.tolenex_logits(toks, as_f64(w), cfg), F32_TOL, f'{n} tokens one by one')
 
 
-def test_long_decoding():
-    cfg = make_config([attention_layer(ff=0), hgrn2_layer(ff=40)], loop=(0, 2, 2))
+@pytest.mark.parametrize('stack', sorted(STACKS))
+def test_long_decoding(stack):
+    cfg = make_config([STACKS[stack][0], hgrn2_layer(ff=40)], loop=(0, 2, 2))
     w = random_weights(cfg, seed=15)
     toks = tokens_for(cfg, 330, 9)
     want = O.tolenex_logits(toks, as_f64(w), cfg)

@@ -62,7 +62,8 @@ int launch_stack_gelu_gate(void* y, const void* gu, int32_t dtype, int32_t token
 // ---------------------------------------------------------------------------------------------
 // Rotary positions: pair (2i, 2i + 1) of the first `dims` dimensions of every map of every head, angle = pos * freq[i]
 // (fp32), cos / sin scaled by `mscale`; freq carries whatever frequency scaling the model uses (host: stack_rope_freqs).
-// Paged cache of one attention layer: K pool [blocks, kv_heads * maps, page, dim], V pool [blocks, kv_heads, page, vdim].
+// Paged cache of one attention layer: K pool [blocks, kv_heads * maps, page, dim], V pool [blocks, kv_heads, vdim, page] (values
+// channel-major inside a page: the MFMA kernel reads V^T rows).
 // ---------------------------------------------------------------------------------------------
 struct StackAttnParams
 {

@@ -174,7 +174,7 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(const StackAttnParams p)
     for (int i = threadIdx.x; i < nv; i += blockDim.x)
     {
         const int g = i / p.vdim, c = i % p.vdim;
-        El<DT>::st(p.v_pool, (((int64_t) blk * p.kv_heads + g) * p.page + off) * p.vdim + c, El<DT>::ld(p.proj, row + nq + nk + i));
+        El<DT>::st(p.v_pool, (((int64_t) blk * p.kv_heads + g) * p.vdim + c) * p.page + off, El<DT>::ld(p.proj, row + nq + nk + i));
     }
 }
 
@@ -265,7 +265,7 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
                 a[m] = acc[m][c] * corr[m];
             for (int j = 0; j < nb; ++j)
             {
-                const float v = El<DT>::ld(p.v_pool, (((int64_t) blk_of[j] * p.kv_heads + g) * p.page + (k0 + j) % p.page) * V + ch);
+                const float v = El<DT>::ld(p.v_pool, (((int64_t) blk_of[j] * p.kv_heads + g) * V + ch) * p.page + (k0 + j) % p.page);
 #pragma unroll
                 for (int m = 0; m < MAPS; ++m)
                     a[m] += ps[m * AT + j] * v;
