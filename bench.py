@@ -672,8 +672,6 @@ def main():
     world = int(os.environ.get('WORLD_SIZE', '1'))
     rank = int(os.environ.get('RANK', '0'))
     local = int(os.environ.get('LOCAL_RANK', '0'))
-    if not torch.cuda.is_available():
-        raise SystemExit('bench.py needs a GPU (the HIP path has no CPU fallback)')
     if args.gpus > 1 and 'RANK' not in os.environ:
         # `python bench.py --gpus N` without a launcher: become the launcher - one process per GPU under torch.distributed.run
         # (the reference's model is the same, one process per GPU under mpirun: PY/_utils.py:181-190, Q/run.py:83-93)
@@ -689,7 +687,12 @@ def main():
         cmd = [sys.executable, '-m', 'torch.distributed.run', '--nnodes=1', f'--nproc-per-node={args.gpus}', '--master-addr', '127.0.0.1',
                '--master-port', str(port), os.path.abspath(__file__)] + sys.argv[1:]
         print('[bench] re-launching as: ' + ' '.join(cmd), file=sys.stderr, flush=True)
-        os.execv(sys.executable, cmd)
+        # a child process, and before anything here has touched the GPU (device_count() does not initialise it): a process that
+        # holds the GPU must not replace itself with another program
+        import subprocess
+        raise SystemExit(subprocess.run(cmd).returncode)
+    if not torch.cuda.is_available():
+        raise SystemExit('bench.py needs a GPU (the HIP path has no CPU fallback)')
     if world != args.gpus:
         raise SystemExit(f'bench.py --gpus {args.gpus} inside a launcher of WORLD_SIZE {world}: start it with --nproc-per-node {args.gpus}')
     if os.environ.get('TLLM_TEST_SHARED_GPU') == '1':

@@ -369,6 +369,99 @@ __global__ __launch_bounds__(64) void hgrn2_scan_kernel(const StackHgrnParams p)
     }
 }
 
+// The head-wide form: one workgroup per (entry, head) when the head's vdim channels fit one workgroup (<= 256).  Thread v keeps
+// column S[:, v] in registers; rows go through in chunks of HTC: the chunk's gates and queries are computed once per (row, channel
+// of dim) and its values fetched, all loads of the chunk in flight together, then the recurrence walks the chunk out of LDS, and the
+// per-head RMS norm of the chunk's outputs is taken in the same launch (no fp32 round trip of o, no second kernel).
+constexpr int HTC = 16;
+
+template <int DT, int DMAX, int NT>
+__global__ __launch_bounds__(NT) void hgrn2_head_kernel(const StackHgrnParams p)
+{
+    __shared__ float2 fq[HTC][DMAX]; // {forget gate, query}
+    __shared__ float vs[HTC][NT];
+    __shared__ float os[HTC][NT];
+    __shared__ float red[HTC][NT / 64];
+    const int e = blockIdx.x, h = blockIdx.y, v = threadIdx.x, lane = v & 63, wid = v >> 6;
+    const int D = p.dim, V = p.vdim, HD = p.heads * D;
+    const int first = p.ent_first[e], count = p.ent_count[e];
+    const bool live = v < V;
+    float* sp = p.state + (((int64_t) p.ent_slot[e] * p.heads + h) * D) * V + v;
+    const bool carry = p.ent_pos0[e] > 0;
+    float S[DMAX];
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d)
+        S[d] = (live && d < D && carry) ? sp[(int64_t) d * V] : 0.f;
+    const float nw = live ? p.norm_w[v] : 0.f;
+    for (int t0 = 0; t0 < count; t0 += HTC)
+    {
+        const int nt = count - t0 < HTC ? count - t0 : HTC;
+        __syncthreads();
+        for (int i = v; i < nt * D; i += NT)
+        {
+            const int tt = i / D, d = i % D;
+            const int64_t row = (int64_t) (first + t0 + tt) * p.ldp;
+            float qr = El<DT>::ld(p.proj, row + h * D + d);
+            qr = qr / (1.f + expf(-qr));
+            if (DT == DT_BF16)
+                qr = bf2f(f2bf(qr)); // the projection's activation is a bfloat16 value; everything behind it is fp32
+            const float fr = El<DT>::ld(p.proj, row + HD + h * D + d) + p.f_bias[h * D + d];
+            const float lo = p.lower[h * D + d];
+            fq[tt][d] = make_float2(lo + (1.f - lo) * (1.f / (1.f + expf(-fr))), qr);
+        }
+        float vv[HTC];
+#pragma unroll
+        for (int tt = 0; tt < HTC; ++tt)
+            vv[tt] = (live && tt < nt) ? El<DT>::ld(p.proj, (int64_t) (first + t0 + tt) * p.ldp + 2 * HD + h * V + v) : 0.f;
+#pragma unroll
+        for (int tt = 0; tt < HTC; ++tt)
+            vs[tt][v] = vv[tt];
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt)
+        {
+            const float x = vs[tt][v];
+            float o = 0.f;
+#pragma unroll
+            for (int d = 0; d < DMAX; ++d)
+            {
+                if (d < D)
+                {
+                    const float2 c = fq[tt][d];
+                    S[d] = c.x * S[d] + (1.f - c.x) * x;
+                    o += S[d] * c.y;
+                }
+            }
+            os[tt][v] = live ? o : 0.f;
+        }
+        for (int tt = 0; tt < nt; ++tt)
+        {
+            const float o = os[tt][v];
+            const float ss = wave_sum(o * o);
+            if (lane == 0)
+                red[tt][wid] = ss;
+        }
+        __syncthreads();
+        if (live)
+        {
+            for (int tt = 0; tt < nt; ++tt)
+            {
+                float ss = 0.f;
+#pragma unroll
+                for (int w = 0; w < NT / 64; ++w)
+                    ss += red[tt][w];
+                El<DT>::st(p.out, (int64_t) (first + t0 + tt) * (p.heads * V) + h * V + v, os[tt][v] * (1.f / sqrtf(ss / (float) V + p.eps)) * nw);
+            }
+        }
+    }
+    if (live)
+    {
+#pragma unroll
+        for (int d = 0; d < DMAX; ++d)
+            if (d < D)
+                sp[(int64_t) d * V] = S[d];
+    }
+}
+
 // per (row, head): o / sqrt(mean(o^2) + eps) * w over the head's vdim channels; one wave each
 template <int DT>
 __global__ __launch_bounds__(256) void head_rmsnorm_kernel(void* y, const float* o, const float* w, int64_t n_heads_total, int vdim, float eps)
@@ -548,6 +641,39 @@ int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
         set_error("stack_hgrn2: heads %d, dim %d, vdim %d is not a shape it serves (dim <= 128: a state column lives in registers)", p.heads,
             p.dim, p.vdim);
         return -1;
+    }
+    if (p.vdim <= 256)
+    {
+        const dim3 hg(p.entries, p.heads);
+#define TLLM_HGRN_H(DT, DMAX)                                                                                                   \
+    do                                                                                                                              \
+    {                                                                                                                               \
+        if (p.vdim <= 64)                                                                                                           \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, DMAX, 64>), hg, dim3(64), 0, stream, p);                                      \
+        else if (p.vdim <= 128)                                                                                                     \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, DMAX, 128>), hg, dim3(128), 0, stream, p);                                    \
+        else                                                                                                                        \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, DMAX, 256>), hg, dim3(256), 0, stream, p);                                    \
+    } while (0)
+#define TLLM_HGRN_HD(DT)                                                                                                        \
+    do                                                                                                                              \
+    {                                                                                                                               \
+        if (p.dim <= 16)                                                                                                            \
+            TLLM_HGRN_H(DT, 16);                                                                                                    \
+        else if (p.dim <= 32)                                                                                                       \
+            TLLM_HGRN_H(DT, 32);                                                                                                    \
+        else if (p.dim <= 64)                                                                                                       \
+            TLLM_HGRN_H(DT, 64);                                                                                                    \
+        else                                                                                                                        \
+            TLLM_HGRN_H(DT, 128);                                                                                                   \
+    } while (0)
+        if (p.dtype == DT_BF16)
+            TLLM_HGRN_HD(DT_BF16);
+        else
+            TLLM_HGRN_HD(DT_FLOAT);
+#undef TLLM_HGRN_HD
+#undef TLLM_HGRN_H
+        return launched("stack_hgrn2 (head-wide)");
     }
     const dim3 grid(p.entries, p.heads, (p.vdim + 63) / 64);
 #define TLLM_HGRN(DT, DMAX) hipLaunchKernelGGL((hgrn2_scan_kernel<DT, DMAX>), grid, dim3(64), 0, stream, p)
