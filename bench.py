@@ -66,6 +66,7 @@ def parse():
                     help="tolenex: a side report instead of the headline workload - prefill and decode throughput of the Tolenex design "
                          "(bfloat16, ragged stack engine) at layer sizes of real models, beside LLaMA fp16 at equal size")
     ap.add_argument('--design-sizes', default='2048,4096', help='--design tolenex: comma list of model widths')
+    ap.add_argument('--design-no-llama', action='store_true', help='--design tolenex: skip the LLaMA side (kernel traces of the new design alone)')
     ap.add_argument('--design-layers', type=int, default=4, help='--design tolenex: layers of both models')
     ap.add_argument('--cpu-sweep', default='', help='debug: comma list of thread counts to try (stderr)')
     return ap.parse_args()
@@ -629,6 +630,9 @@ def tolenex_report(torch, args, dev):
             ctx = sess.length_of('p')
             row[f'tolenex_decode_b{batch}_hbm_fraction'] = sess.engine.step_bytes(batch, batch * ctx, batch) / (dt / K) / 8e12
         del sess, model
+        if args.design_no_llama:
+            rows.append({k: (round(v, 3) if isinstance(v, float) else v) for k, v in row.items()})
+            continue
         # LLaMA fp16 at equal size
         lc = dict(num_layers=L, num_heads=width // 128, hidden_size=width, inter_size=int(width * 2.6875), vocab_size=cfg['vocab'],
                   max_position_embeddings=S + 2 * K + 2 * W + 64, rms_norm_eps=1e-5, quant_mode=0)

@@ -1,11 +1,14 @@
 // Products of the stack engine (stack_kernels.h): C[m,n] = sum_k A[m,k] * W[n,k] with the layer seam in the epilogue.
 //
-//   bfloat16, M > 8 : MFMA tiles of gemm_mfma.hip (v_mfma_f32_32x32x16_bf16);
+//   bfloat16, M >= 32, K % 64 == 0: the LDS-DMA staged MFMA tiles of gemm_glds_impl.h instantiated for bfloat16 operands
+//                     (v_mfma_f32_32x32x16_bf16), tile shape by the same rounds x area rule as the fp16 form;
+//   bfloat16, other M > 8: the register-staged MFMA tiles of gemm_mfma.hip;
 //   bfloat16, M <= 8: skinny_kernel below - HBM-bound, a wave streams R weight rows with 16-byte non-temporal loads and keeps the
 //                     M activation rows' chunks in registers; fp32 accumulation, DPP reduction;
 //   float32         : fma_tile_kernel - 64 x 64 tiles of plain fp32 FMAs through LDS (no reduced-precision matrix mode), any shape;
 //                     also the fallback for bfloat16 operands whose rows are not 16-byte aligned.
 #include "dev_utils.h"
+#include "gemm_glds_impl.h"
 #include "stack_kernels.h"
 
 namespace tllm
@@ -167,6 +170,38 @@ inline int launched(const char* what)
     return 0;
 }
 
+// the lock-step tile shapes of the LDS-DMA kernel and what a tile of each kind costs per area (measured on fp16 operands; the
+// bfloat16 MFMA has the same rate and byte geometry): fewest workgroup rounds x area x cost
+int launch_glds_bf16(const GemmParams& g, hipStream_t stream)
+{
+    struct Shape
+    {
+        int id, bm, bn;
+        double f;
+    };
+    static const Shape shapes[] = {{0, 128, 128, 1.40}, {1, 256, 192, 1.0}, {2, 256, 256, 1.04}, {3, 128, 256, 1.39}};
+    const int cus = launch_util::device_cus();
+    double best = 1e30;
+    int pick = 0;
+    for (const Shape& sh : shapes)
+    {
+        const int64_t tiles = (int64_t) ((g.M + sh.bm - 1) / sh.bm) * ((g.N + sh.bn - 1) / sh.bn);
+        const double cost = (double) ((tiles + cus - 1) / cus) * sh.bm * sh.bn * sh.f;
+        if (cost < best)
+        {
+            best = cost;
+            pick = sh.id;
+        }
+    }
+    switch (pick)
+    {
+    case 1: return launch_cfg<W_BF16, 4, 2, 2, 3, 1, 64, 5>(g, stream);
+    case 2: return launch_cfg<W_BF16, 2, 4, 4, 2, 1, 64, 4>(g, stream);
+    case 3: return launch_cfg<W_BF16, 2, 2, 2, 4, 1, 64, 4>(g, stream);
+    default: return launch_cfg<W_BF16, 2, 2, 2, 2, 1, 128, 4>(g, stream);
+    }
+}
+
 } // namespace
 
 int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
@@ -220,6 +255,8 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
         g.gate = p.gate;
         g.ldg = p.ldg;
         g.gate_bias = p.gate_bias;
+        if (p.M >= 32 && p.K % 64 == 0)
+            return launch_glds_bf16(g, stream);
         const int rc = launch_gemm_mfma(g, stream);
         if (rc <= 0)
             return rc;
