@@ -12,6 +12,7 @@
 #include "dev_utils.h"
 #include "launch_util.h"
 #include "stack_kernels.h"
+#include <cstdlib>
 
 namespace tllm
 {
@@ -33,8 +34,82 @@ __device__ __forceinline__ bf16x8 as_bf16x8(const uint4& u)
     return r;
 }
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// max / sum over the four lanes that hold the same query row (lane ^ 16, lane ^ 32)
+__device__ __forceinline__ float rows_max(float v)
+{
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    return fmaxf(v, __shfl_xor(v, 32, 64));
+}
+__device__ __forceinline__ float rows_sum(float v)
+{
+    v += __shfl_xor(v, 16, 64);
+    return v + __shfl_xor(v, 32, 64);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
+{
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
+
+// Scores of one 32-key block of one map -> its P^T fragment, with the online-softmax state of the lane's query row brought up to
+// date.  Everything in the base-2 domain (scale2 / cap2 carry log2 e), so an exponential is one v_exp_f32.  `masked` is wave-uniform:
+// only blocks that reach past the first row's position compare keys with positions.
+template <int VT>
+__device__ __forceinline__ uint4 softmax_block(f32x4 (&s)[2], float& m_run, float& l_run, f32x4 (&acc)[VT], float scale2, float cap2,
+    float cap_arg, bool masked, int key_lane0, int qpos)
+{
+    float bm = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            float v;
+            if (cap2 > 0.f)
+            {
+                // cap * tanh(x / cap) with tanh(y) = (e^{2y} - 1) / (e^{2y} + 1); cap_arg = scale / cap * 2 log2 e
+                const float t2 = __builtin_amdgcn_exp2f(fminf(fmaxf(s[t][i] * cap_arg, -43.f), 43.f));
+                v = cap2 * (t2 - 1.f) * __builtin_amdgcn_rcpf(t2 + 1.f);
+            }
+            else
+                v = s[t][i] * scale2;
+            if (masked && key_lane0 + t * 16 + i > qpos)
+                v = -INFINITY;
+            s[t][i] = v;
+            bm = fmaxf(bm, v);
+        }
+    bm = rows_max(bm);
+    const float mn = fmaxf(m_run, bm);
+    const bool none = mn == -INFINITY; // this row sees no key of this block (nor of any before)
+    const float corr = none ? 1.f : __builtin_amdgcn_exp2f(m_run - mn);
+    float rs = 0.f, pv[8];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            pv[t * 4 + i] = none ? 0.f : __builtin_amdgcn_exp2f(s[t][i] - mn);
+            rs += pv[t * 4 + i];
+        }
+    rs = rows_sum(rs);
+    l_run = l_run * corr + rs;
+    m_run = mn;
+    // the accumulators are rescaled only when some row's maximum moved (wave-uniform test): behind the first blocks of a long
+    // context it rarely does, and the accumulators sit in the matrix pipe's registers, a round trip per element away
+    if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0)
+    {
+#pragma unroll
+        for (int ct = 0; ct < VT; ++ct)
+            acc[ct] *= corr;
+    }
+    return make_uint4(pack_bf16(pv[0], pv[1]), pack_bf16(pv[2], pv[3]), pack_bf16(pv[4], pv[5]), pack_bf16(pv[6], pv[7]));
+}
+
 template <int MAPS, int DK, int VT, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParams p)
+__global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParams p, int below_count)
 {
     constexpr int D = DK * 32, V = VT * 16;
     extern __shared__ float lds[];
@@ -42,7 +117,7 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     float* ml_part = lds + NW * MAPS * 16 * V;    // [NW][MAPS][16][2]
     const int e = blockIdx.y, h = blockIdx.z, r0 = blockIdx.x * 16;
     const int count = p.ent_count[e];
-    if (r0 >= count)
+    if (r0 >= count || count >= below_count) // entries of below_count rows and more are the prefill form's
         return;
     const int first = p.ent_first[e], pos0 = p.ent_pos0[e];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -50,6 +125,9 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     const int g = h / (p.heads / p.kv_heads);
     const int page = p.page;
     const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float scale2 = p.scale * LOG2E, cap2 = p.softcap > 0.f ? p.softcap * LOG2E : 0.f;
+    const float cap_arg = p.softcap > 0.f ? p.scale / p.softcap * 2.f * LOG2E : 0.f;
     const uint16_t* kp = reinterpret_cast<const uint16_t*>(p.k_pool);
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.v_pool);
 
@@ -77,73 +155,64 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
             acc[m][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    for (int kb = w; kb < nblk; kb += NW)
-    {
-        const int key0 = kb * 32;
-        const int blk = table[key0 / page], off = key0 % page;
-        uint4 pf[MAPS]; // P^T fragment of the block, 8 bfloat16 per map
+    // Software pipeline: the K fragments of a block are requested one iteration ahead, its V^T fragments at the top of its own
+    // iteration, so that the score / softmax arithmetic of a block (the long part: it is all VALU) runs with both in flight.
+    uint4 kf[MAPS][2][DK];
+    auto request_k = [&](int kb, int blk) {
+        const int off = (kb * 32) % page;
 #pragma unroll
         for (int m = 0; m < MAPS; ++m)
-        {
-            f32x4 s[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
             {
-                s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
                 const uint16_t* krow = kp + (((int64_t) blk * (p.kv_heads * MAPS) + g * MAPS + m) * page + off + t * 16 + col) * D + 8 * g4;
 #pragma unroll
                 for (int ks = 0; ks < DK; ++ks)
-                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(*reinterpret_cast<const uint4*>(krow + ks * 32)), qf[m][ks],
-                        s[t], 0, 0, 0);
+                    kf[m][t][ks] = *reinterpret_cast<const uint4*>(krow + ks * 32);
             }
-            float bm = -INFINITY;
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                {
-                    float v = s[t][i] * p.scale;
-                    if (p.softcap > 0.f)
-                        v = p.softcap * tanhf(v / p.softcap);
-                    if (key0 + t * 16 + 4 * g4 + i > qpos)
-                        v = -INFINITY;
-                    s[t][i] = v;
-                    bm = fmaxf(bm, v);
-                }
-            bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
-            bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
-            const float mn = fmaxf(m_run[m], bm);
-            const bool none = mn == -INFINITY; // this row sees no key of this block (nor of any before)
-            const float corr = none ? 1.f : __expf(m_run[m] - mn);
-            float rs = 0.f;
-            float pv[8];
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                {
-                    const float e_ = none ? 0.f : __expf(s[t][i] - mn);
-                    pv[t * 4 + i] = e_;
-                    rs += e_;
-                }
-            rs += __shfl_xor(rs, 16, 64);
-            rs += __shfl_xor(rs, 32, 64);
-            l_run[m] = l_run[m] * corr + rs;
-            m_run[m] = mn;
+    };
+    int blk = w < nblk ? table[w * 32 / page] : 0;
+    if (w < nblk)
+        request_k(w, blk);
+    for (int kb = w; kb < nblk; kb += NW)
+    {
+        const int key0 = kb * 32, off = key0 % page;
+        uint2 vlo[VT], vhi[VT];
+        {
+            const uint16_t* vrow = vp + (((int64_t) blk * p.kv_heads + g) * V + col) * page + off + 4 * g4;
 #pragma unroll
             for (int ct = 0; ct < VT; ++ct)
-                acc[m][ct] *= corr;
-            pf[m] = make_uint4((uint32_t) f2bf(pv[0]) | ((uint32_t) f2bf(pv[1]) << 16), (uint32_t) f2bf(pv[2]) | ((uint32_t) f2bf(pv[3]) << 16),
-                (uint32_t) f2bf(pv[4]) | ((uint32_t) f2bf(pv[5]) << 16), (uint32_t) f2bf(pv[6]) | ((uint32_t) f2bf(pv[7]) << 16));
+            {
+                vlo[ct] = *reinterpret_cast<const uint2*>(vrow + (int64_t) ct * 16 * page);
+                vhi[ct] = *reinterpret_cast<const uint2*>(vrow + (int64_t) ct * 16 * page + 16);
+            }
         }
+        f32x4 s[MAPS][2];
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+            {
+                s[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < DK; ++ks)
+                    s[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[m][t][ks]), qf[m][ks], s[m][t], 0, 0, 0);
+            }
+        if (kb + NW < nblk)
+        {
+            blk = table[(key0 + NW * 32) / page];
+            request_k(kb + NW, blk);
+        }
+        uint4 pf[MAPS]; // P^T fragment of the block, 8 bfloat16 per map
+        const bool masked = key0 + 31 > pos0 + r0; // wave-uniform
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m)
+            pf[m] = softmax_block<VT>(s[m], m_run[m], l_run[m], acc[m], scale2, cap2, cap_arg, masked, key0 + 4 * g4, qpos);
         // O^T += V^T P^T: slot j of the lane's k group is key 4 g4 + j (j < 4) or 16 + 4 g4 + (j - 4) of the block, in both operands
-        const uint16_t* vrow = vp + (((int64_t) blk * p.kv_heads + g) * V + col) * page + off + 4 * g4;
 #pragma unroll
         for (int ct = 0; ct < VT; ++ct)
         {
-            const uint2 lo = *reinterpret_cast<const uint2*>(vrow + (int64_t) ct * 16 * page);
-            const uint2 hi = *reinterpret_cast<const uint2*>(vrow + (int64_t) ct * 16 * page + 16);
-            const bf16x8 vf = as_bf16x8(make_uint4(lo.x, lo.y, hi.x, hi.y));
+            const bf16x8 vf = as_bf16x8(make_uint4(vlo[ct].x, vlo[ct].y, vhi[ct].x, vhi[ct].y));
 #pragma unroll
             for (int m = 0; m < MAPS; ++m)
                 acc[m][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, as_bf16x8(pf[m]), acc[m][ct], 0, 0, 0);
@@ -182,7 +251,7 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
         for (int ww = 0; ww < NW; ++ww)
         {
             const float mw = ml_part[((ww * MAPS + m) * 16 + row) * 2];
-            wgt[m][ww] = mw == -INFINITY ? 0.f : __expf(mw - M);
+            wgt[m][ww] = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M); // the running maxima are base-2 exponents
             L += wgt[m][ww] * ml_part[((ww * MAPS + m) * 16 + row) * 2 + 1];
         }
 #pragma unroll
@@ -229,6 +298,184 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     }
 }
 
+// attn_prefill_kernel: the form for entries that bring many rows.  One workgroup per (64 rows of an entry, head), wave w owns rows
+// 16 w .. 16 w + 15; all four waves walk the same 32-key blocks, which the workgroup stages once through LDS (K rows padded to an odd
+// number of 16-byte pieces, V^T rows to 80 bytes: the fragment reads spread over the banks) - the next block's global loads are in
+// flight while this block is computed.  Same transposed products and operand slots as attn_tile_kernel; no merge: a wave finishes
+// its own rows (lambda combination, head norm, bfloat16 store).  Tiles are handed out heaviest first (the last rows see most keys).
+template <int MAPS, int DK, int VT>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams p, int min_count)
+{
+    constexpr int D = DK * 32, V = VT * 16;
+    constexpr int KP = D * 2 + 16, VP = 80;                 // LDS row pitches in bytes
+    constexpr int K16 = MAPS * 32 * (D / 8), V16 = V * 4;   // 16-byte pieces per block
+    constexpr int KPT = (K16 + 255) / 256, VPT = (V16 + 255) / 256;
+    __shared__ __attribute__((aligned(16))) char k_s[MAPS * 32 * KP];
+    __shared__ __attribute__((aligned(16))) char v_s[V * VP];
+    const int e = blockIdx.y, h = blockIdx.z;
+    const int count = p.ent_count[e];
+    if (count < min_count)
+        return;
+    const int tile = (count + 63) / 64 - 1 - (int) blockIdx.x;
+    if (tile < 0)
+        return;
+    const int first = p.ent_first[e], pos0 = p.ent_pos0[e];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int col = lane & 15, g4 = lane >> 4;
+    const int g = h / (p.heads / p.kv_heads);
+    const int page = p.page;
+    const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float scale2 = p.scale * LOG2E, cap2 = p.softcap > 0.f ? p.softcap * LOG2E : 0.f;
+    const float cap_arg = p.softcap > 0.f ? p.scale / p.softcap * 2.f * LOG2E : 0.f;
+    const uint16_t* kp = reinterpret_cast<const uint16_t*>(p.k_pool);
+    const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.v_pool);
+
+    const int r0 = tile * 64 + w * 16;
+    const bool wave_rows = r0 < count; // wave-uniform
+    const int qrow = r0 + col < count ? r0 + col : count - 1;
+    const int qpos = pos0 + qrow;
+    bf16x8 qf[MAPS][DK];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks)
+            qf[m][ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
+                reinterpret_cast<const uint16_t*>(p.q) + (((int64_t) (first + qrow) * p.heads + h) * MAPS + m) * D + ks * 32 + 8 * g4));
+    const int wg_last = tile * 64 + 63 < count ? tile * 64 + 63 : count - 1;
+    const int nblk = (pos0 + wg_last) / 32 + 1;
+    const int my_last = r0 + 15 < count ? r0 + 15 : count - 1;
+    const int my_blk = wave_rows ? (pos0 + my_last) / 32 : -1; // the wave's last block that holds a visible key
+
+    float m_run[MAPS], l_run[MAPS];
+    f32x4 acc[MAPS][VT];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+    {
+        m_run[m] = -INFINITY;
+        l_run[m] = 0.f;
+#pragma unroll
+        for (int ct = 0; ct < VT; ++ct)
+            acc[m][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    uint4 kr[KPT], vr[VPT];
+    // the page id of a block is fetched one block before its rows are requested: one memory latency per block, not two in a row
+    int blk_next = table[0];
+    auto request = [&](int kb) {
+        const int key0 = kb * 32;
+        const int blk = blk_next, off = key0 % page;
+        blk_next = table[kb + 1 < nblk ? (key0 + 32) / page : key0 / page];
+#pragma unroll
+        for (int i = 0; i < KPT; ++i)
+        {
+            const int idx = tid + i * 256;
+            if (K16 % 256 == 0 || idx < K16)
+            {
+                const int row = idx / (D / 8), piece = idx % (D / 8); // row = map * 32 + key
+                kr[i] = *reinterpret_cast<const uint4*>(
+                    kp + (((int64_t) blk * (p.kv_heads * MAPS) + g * MAPS + row / 32) * page + off + row % 32) * D + piece * 8);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; ++i)
+        {
+            const int idx = tid + i * 256;
+            if (V16 % 256 == 0 || idx < V16)
+                vr[i] = *reinterpret_cast<const uint4*>(vp + (((int64_t) blk * p.kv_heads + g) * V + idx / 4) * page + off + (idx % 4) * 8);
+        }
+    };
+    request(0);
+    for (int kb = 0; kb < nblk; ++kb)
+    {
+#pragma unroll
+        for (int i = 0; i < KPT; ++i)
+        {
+            const int idx = tid + i * 256;
+            if (K16 % 256 == 0 || idx < K16)
+                *reinterpret_cast<uint4*>(k_s + (idx / (D / 8)) * KP + (idx % (D / 8)) * 16) = kr[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; ++i)
+        {
+            const int idx = tid + i * 256;
+            if (V16 % 256 == 0 || idx < V16)
+                *reinterpret_cast<uint4*>(v_s + (idx / 4) * VP + (idx % 4) * 16) = vr[i];
+        }
+        __syncthreads();
+        if (kb + 1 < nblk)
+            request(kb + 1);
+        if (kb <= my_blk)
+        {
+            const int key0 = kb * 32;
+            uint4 pf[MAPS];
+            const bool masked = key0 + 31 > pos0 + r0; // wave-uniform
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m)
+            {
+                f32x4 s[2];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                {
+                    s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < DK; ++ks)
+                        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            as_bf16x8(*reinterpret_cast<const uint4*>(k_s + (m * 32 + t * 16 + col) * KP + (ks * 32 + 8 * g4) * 2)), qf[m][ks], s[t],
+                            0, 0, 0);
+                }
+                pf[m] = softmax_block<VT>(s, m_run[m], l_run[m], acc[m], scale2, cap2, cap_arg, masked, key0 + 4 * g4, qpos);
+            }
+#pragma unroll
+            for (int ct = 0; ct < VT; ++ct)
+            {
+                const char* vrow = v_s + (ct * 16 + col) * VP + 8 * g4;
+                const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+                const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 32);
+                const bf16x8 vf = as_bf16x8(make_uint4(lo.x, lo.y, hi.x, hi.y));
+#pragma unroll
+                for (int m = 0; m < MAPS; ++m)
+                    acc[m][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, as_bf16x8(pf[m]), acc[m][ct], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    if (!wave_rows)
+        return;
+    // lane (col, g4) holds, for row col, channels ct * 16 + 4 g4 + i
+    float inv[MAPS];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+        inv[m] = 1.f / l_run[m];
+    float ss = 0.f;
+#pragma unroll
+    for (int ct = 0; ct < VT; ++ct)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            float o = acc[0][ct][i] * inv[0];
+            if (MAPS == 2)
+                o -= p.lambda * (acc[MAPS - 1][ct][i] * inv[MAPS - 1]);
+            acc[0][ct][i] = o;
+            ss += o * o;
+        }
+    float mul = 1.f;
+    if (p.head_norm)
+    {
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        mul = p.out_scale / sqrtf(ss / (float) V + p.eps);
+    }
+    if (r0 + col < count)
+    {
+        uint16_t* out = reinterpret_cast<uint16_t*>(p.out) + ((int64_t) (first + r0 + col) * p.heads + h) * V + 4 * g4;
+#pragma unroll
+        for (int ct = 0; ct < VT; ++ct)
+            *reinterpret_cast<uint2*>(out + ct * 16) = make_uint2((uint32_t) f2bf(acc[0][ct][0] * mul) | ((uint32_t) f2bf(acc[0][ct][1] * mul) << 16),
+                (uint32_t) f2bf(acc[0][ct][2] * mul) | ((uint32_t) f2bf(acc[0][ct][3] * mul) << 16));
+    }
+}
+
 template <int MAPS, int DK, int VT>
 int launch_tile(const StackAttnParams& p, hipStream_t stream)
 {
@@ -236,12 +483,27 @@ int launch_tile(const StackAttnParams& p, hipStream_t stream)
     const size_t lds = sizeof(float) * ((size_t) NW * MAPS * 16 * VT * 16 + (size_t) NW * MAPS * 16 * 2);
     const void* fn = reinterpret_cast<const void*>(&attn_tile_kernel<MAPS, DK, VT, NW>);
     launch_util::ensure_dynamic_lds(fn, lds);
-    const dim3 grid((p.max_count + 15) / 16, p.entries, p.heads);
-    hipLaunchKernelGGL((attn_tile_kernel<MAPS, DK, VT, NW>), grid, dim3(NW * 64), lds, stream, p);
+    // entries of PREFILL_ROWS rows and more go to the staged form, the rest (decoded tokens, short portions) to the key-split form;
+    // a mixed step launches both, each skipping the other's entries
+    static const int PREFILL_ROWS = [] {
+        const char* v = std::getenv("TLLM_STACK_PREFILL_ROWS"); // measurement knob: rows from which an entry takes the staged form
+        return v && std::atoi(v) > 0 ? std::atoi(v) : 32;
+    }();
+    const int small_rows = p.max_count < PREFILL_ROWS ? p.max_count : (p.tokens > p.max_count ? PREFILL_ROWS - 1 : 0);
+    if (p.max_count >= PREFILL_ROWS)
+    {
+        const dim3 pg((p.max_count + 63) / 64, p.entries, p.heads);
+        hipLaunchKernelGGL((attn_prefill_kernel<MAPS, DK, VT>), pg, dim3(256), 0, stream, p, PREFILL_ROWS);
+    }
+    if (small_rows > 0)
+    {
+        const dim3 grid((small_rows + 15) / 16, p.entries, p.heads);
+        hipLaunchKernelGGL((attn_tile_kernel<MAPS, DK, VT, NW>), grid, dim3(NW * 64), lds, stream, p, PREFILL_ROWS);
+    }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess)
     {
-        set_error("stack_attention (tile kernel) launch failed: %s", hipGetErrorString(e));
+        set_error("stack_attention (tile kernels) launch failed: %s", hipGetErrorString(e));
         return -1;
     }
     return 0;

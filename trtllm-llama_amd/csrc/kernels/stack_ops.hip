@@ -3,6 +3,7 @@
 // activations, weights and caches (bfloat16 or fp32).
 #include "dev_utils.h"
 #include "stack_kernels.h"
+#include <algorithm>
 #include <cmath>
 #include <vector>
 
@@ -93,31 +94,49 @@ __global__ __launch_bounds__(256) void pass_entry_kernel(float* x, const float* 
     x[i] = v;
 }
 
-// one workgroup per row, wave w takes groups w, w + waves, ...: no workgroup barrier
+// one workgroup per (row, group): the group's elements stay in registers between the sum of squares and the scaling
+constexpr int GN_T = 256, GN_EPT = 8;
+
 template <int DT>
-__global__ __launch_bounds__(256) void group_rmsnorm_kernel(void* y1, void* y2, const float* x, const int32_t* rows, const float* w1,
+__global__ __launch_bounds__(GN_T) void group_rmsnorm_kernel(void* y1, void* y2, const float* x, const int32_t* rows, const float* w1,
     const float* w2, int width, int groups, float eps)
 {
-    const int r = blockIdx.x;
-    const float* xr = x + (int64_t) (rows ? rows[r] : r) * width;
-    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __shared__ float red[32];
+    const int r = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
     const int gs = width / groups;
-    for (int g = wid; g < groups; g += nw)
+    const float* xg = x + (int64_t) (rows ? rows[r] : r) * width + g * gs;
+    float v[GN_EPT], ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < GN_EPT; ++k)
     {
-        const float* xg = xr + g * gs;
-        float ss = 0.f;
-        for (int i = lane; i < gs; i += 64)
-            ss += xg[i] * xg[i];
-        ss = wave_sum(ss);
-        const float inv = 1.f / sqrtf(ss / (float) gs + eps);
-        for (int i = lane; i < gs; i += 64)
+        const int i = tid + k * GN_T;
+        v[k] = i < gs ? xg[i] : 0.f;
+        ss += v[k] * v[k];
+    }
+    for (int i = tid + GN_EPT * GN_T; i < gs; i += GN_T) // groups beyond GN_T * GN_EPT elements: the tail is read twice
+        ss += xg[i] * xg[i];
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float) gs + eps);
+#pragma unroll
+    for (int k = 0; k < GN_EPT; ++k)
+    {
+        const int i = tid + k * GN_T;
+        if (i < gs)
         {
             const int c = g * gs + i;
-            const float n = xg[i] * inv;
+            const float n = v[k] * inv;
             El<DT>::st(y1, (int64_t) r * width + c, n * w1[c]);
             if (y2)
                 El<DT>::st(y2, (int64_t) r * width + c, n * w2[c]);
         }
+    }
+    for (int i = tid + GN_EPT * GN_T; i < gs; i += GN_T)
+    {
+        const int c = g * gs + i;
+        const float n = xg[i] * inv;
+        El<DT>::st(y1, (int64_t) r * width + c, n * w1[c]);
+        if (y2)
+            El<DT>::st(y2, (int64_t) r * width + c, n * w2[c]);
     }
 }
 
@@ -149,7 +168,7 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(const StackAttnParams p)
     const int blk = p.block_table[(int64_t) e * p.max_blocks + pos / p.page], off = pos % p.page;
     const int D = p.dim, nq = p.heads * p.maps * D, nk = p.kv_heads * p.maps * D, nv = p.kv_heads * p.vdim;
     const int64_t row = (int64_t) t * p.ldp;
-    for (int i = threadIdx.x; i < nq + nk; i += blockDim.x)
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < nq + nk; i += gridDim.y * blockDim.x)
     {
         const int d = i % D;
         float v = El<DT>::ld(p.proj, row + i);
@@ -171,7 +190,7 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(const StackAttnParams p)
             El<DT>::st(p.k_pool, (((int64_t) blk * (p.kv_heads * p.maps) + gm) * p.page + off) * D + d, v);
         }
     }
-    for (int i = threadIdx.x; i < nv; i += blockDim.x)
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < nv; i += gridDim.y * blockDim.x)
     {
         const int g = i / p.vdim, c = i % p.vdim;
         El<DT>::st(p.v_pool, (((int64_t) blk * p.kv_heads + g) * p.vdim + c) * p.page + off, El<DT>::ld(p.proj, row + nq + nk + i));
@@ -369,96 +388,131 @@ __global__ __launch_bounds__(64) void hgrn2_scan_kernel(const StackHgrnParams p)
     }
 }
 
-// The head-wide form: one workgroup per (entry, head) when the head's vdim channels fit one workgroup (<= 256).  Thread v keeps
-// column S[:, v] in registers; rows go through in chunks of HTC: the chunk's gates and queries are computed once per (row, channel
-// of dim) and its values fetched, all loads of the chunk in flight together, then the recurrence walks the chunk out of LDS, and the
-// per-head RMS norm of the chunk's outputs is taken in the same launch (no fp32 round trip of o, no second kernel).
-constexpr int HTC = 16;
+// The head-wide form: one workgroup per (entry, head) when the head's vdim channels fit (<= 256).  The state is spread over
+// vpad x DS threads: thread (s, v) keeps the DSZ rows [s DSZ, (s + 1) DSZ) of column S[:, v] in registers (every wave has one s, so
+// the row's gates and queries come out of LDS as broadcasts).  Rows go through in chunks of HTC: the chunk's gates and queries are
+// computed once per (row, channel of dim), its raw projections having been requested while the chunk before it was in the
+// recurrence; the recurrence itself has no cross-lane traffic, the DS partial outputs of a row meet in LDS once per chunk, and the
+// per-head RMS norm of the outputs is taken in the same launch (no fp32 round trip of o, no second kernel).
+constexpr int HTC = 8, H_PPT = 4;
 
-template <int DT, int DMAX, int NT>
-__global__ __launch_bounds__(NT) void hgrn2_head_kernel(const StackHgrnParams p)
+template <int DT, int DSZ>
+__global__ __launch_bounds__(1024) void hgrn2_head_kernel(const StackHgrnParams p, int vpad, int DS)
 {
-    __shared__ float2 fq[HTC][DMAX]; // {forget gate, query}
-    __shared__ float vs[HTC][NT];
-    __shared__ float os[HTC][NT];
-    __shared__ float red[HTC][NT / 64];
-    const int e = blockIdx.x, h = blockIdx.y, v = threadIdx.x, lane = v & 63, wid = v >> 6;
-    const int D = p.dim, V = p.vdim, HD = p.heads * D;
+    extern __shared__ float hsm[];
+    const int D = p.dim, V = p.vdim, HD = p.heads * D, NT = blockDim.x;
+    float2* fq = reinterpret_cast<float2*>(hsm);        // [HTC][D] {forget gate, query}
+    float* vs = hsm + 2 * HTC * D;                      // [HTC][vpad]
+    float* os = vs + HTC * vpad;                        // [HTC][DS][vpad]
+    float* red = os + HTC * DS * vpad;                  // [HTC][vpad / 64]
+    const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int s = tid / vpad, v = tid % vpad, lane = tid & 63, vw = v >> 6, nvw = vpad >> 6;
     const int first = p.ent_first[e], count = p.ent_count[e];
     const bool live = v < V;
+    const int d0 = s * DSZ;
     float* sp = p.state + (((int64_t) p.ent_slot[e] * p.heads + h) * D) * V + v;
     const bool carry = p.ent_pos0[e] > 0;
-    float S[DMAX];
+    float S[DSZ];
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d)
-        S[d] = (live && d < D && carry) ? sp[(int64_t) d * V] : 0.f;
+    for (int j = 0; j < DSZ; ++j)
+        S[j] = (live && d0 + j < D && carry) ? sp[(int64_t) (d0 + j) * V] : 0.f;
     const float nw = live ? p.norm_w[v] : 0.f;
+
+    float rq[H_PPT], rf[H_PPT], rv[HTC];
+    auto request = [&](int t0) {
+        const int nt = count - t0 < HTC ? count - t0 : HTC;
+#pragma unroll
+        for (int k = 0; k < H_PPT; ++k)
+        {
+            const int i = tid + k * NT;
+            rq[k] = rf[k] = 0.f;
+            if (i < nt * D)
+            {
+                const int64_t row = (int64_t) (first + t0 + i / D) * p.ldp;
+                rq[k] = El<DT>::ld(p.proj, row + h * D + i % D);
+                rf[k] = El<DT>::ld(p.proj, row + HD + h * D + i % D);
+            }
+        }
+#pragma unroll
+        for (int tt = 0; tt < HTC; ++tt)
+            rv[tt] = (s == 0 && live && tt < nt) ? El<DT>::ld(p.proj, (int64_t) (first + t0 + tt) * p.ldp + 2 * HD + h * V + v) : 0.f;
+    };
+    request(0);
     for (int t0 = 0; t0 < count; t0 += HTC)
     {
         const int nt = count - t0 < HTC ? count - t0 : HTC;
-        __syncthreads();
-        for (int i = v; i < nt * D; i += NT)
+#pragma unroll
+        for (int k = 0; k < H_PPT; ++k)
         {
-            const int tt = i / D, d = i % D;
-            const int64_t row = (int64_t) (first + t0 + tt) * p.ldp;
-            float qr = El<DT>::ld(p.proj, row + h * D + d);
-            qr = qr / (1.f + expf(-qr));
-            if (DT == DT_BF16)
-                qr = bf2f(f2bf(qr)); // the projection's activation is a bfloat16 value; everything behind it is fp32
-            const float fr = El<DT>::ld(p.proj, row + HD + h * D + d) + p.f_bias[h * D + d];
-            const float lo = p.lower[h * D + d];
-            fq[tt][d] = make_float2(lo + (1.f - lo) * (1.f / (1.f + expf(-fr))), qr);
+            const int i = tid + k * NT;
+            if (i < nt * D)
+            {
+                const int d = i % D;
+                float qr = rq[k] / (1.f + expf(-rq[k]));
+                if (DT == DT_BF16)
+                    qr = bf2f(f2bf(qr)); // the projection's activation is a bfloat16 value; everything behind it is fp32
+                const float lo = p.lower[h * D + d];
+                fq[i] = make_float2(lo + (1.f - lo) * (1.f / (1.f + expf(-(rf[k] + p.f_bias[h * D + d])))), qr);
+            }
         }
-        float vv[HTC];
+        if (s == 0)
+        {
 #pragma unroll
-        for (int tt = 0; tt < HTC; ++tt)
-            vv[tt] = (live && tt < nt) ? El<DT>::ld(p.proj, (int64_t) (first + t0 + tt) * p.ldp + 2 * HD + h * V + v) : 0.f;
-#pragma unroll
-        for (int tt = 0; tt < HTC; ++tt)
-            vs[tt][v] = vv[tt];
+            for (int tt = 0; tt < HTC; ++tt)
+                vs[tt * vpad + v] = rv[tt];
+        }
         __syncthreads();
+        if (t0 + HTC < count)
+            request(t0 + HTC); // in flight under the recurrence
         for (int tt = 0; tt < nt; ++tt)
         {
-            const float x = vs[tt][v];
+            const float x = vs[tt * vpad + v];
             float o = 0.f;
 #pragma unroll
-            for (int d = 0; d < DMAX; ++d)
+            for (int j = 0; j < DSZ; ++j)
             {
-                if (d < D)
+                if (d0 + j < D)
                 {
-                    const float2 c = fq[tt][d];
-                    S[d] = c.x * S[d] + (1.f - c.x) * x;
-                    o += S[d] * c.y;
+                    const float2 c = fq[tt * D + d0 + j];
+                    S[j] = c.x * S[j] + (1.f - c.x) * x;
+                    o += S[j] * c.y;
                 }
             }
-            os[tt][v] = live ? o : 0.f;
-        }
-        for (int tt = 0; tt < nt; ++tt)
-        {
-            const float o = os[tt][v];
-            const float ss = wave_sum(o * o);
-            if (lane == 0)
-                red[tt][wid] = ss;
+            os[(tt * DS + s) * vpad + v] = live ? o : 0.f;
         }
         __syncthreads();
-        if (live)
+        // rows of the chunk are shared out over the slices: thread (s, v) finishes rows s, s + DS, ...
+        for (int tt = s; tt < nt; tt += DS) // wave-uniform
         {
-            for (int tt = 0; tt < nt; ++tt)
+            float o = 0.f;
+            for (int s2 = 0; s2 < DS; ++s2)
+                o += os[(tt * DS + s2) * vpad + v];
+            const float ss = wave_sum(o * o);
+            if (lane == 0)
+                red[tt * nvw + vw] = ss;
+        }
+        __syncthreads();
+        for (int tt = s; tt < nt; tt += DS)
+        {
+            if (live)
             {
-                float ss = 0.f;
-#pragma unroll
-                for (int w = 0; w < NT / 64; ++w)
-                    ss += red[tt][w];
-                El<DT>::st(p.out, (int64_t) (first + t0 + tt) * (p.heads * V) + h * V + v, os[tt][v] * (1.f / sqrtf(ss / (float) V + p.eps)) * nw);
+                float o = 0.f, ss = 0.f;
+                for (int s2 = 0; s2 < DS; ++s2)
+                    o += os[(tt * DS + s2) * vpad + v];
+                for (int w = 0; w < nvw; ++w)
+                    ss += red[tt * nvw + w];
+                El<DT>::st(p.out, (int64_t) (first + t0 + tt) * (p.heads * V) + h * V + v, o * (1.f / sqrtf(ss / (float) V + p.eps)) * nw);
             }
         }
+        // (the next chunk's first write to fq / vs is behind this chunk's last read of them: the barrier above; os and red are
+        // rewritten only behind the next chunk's first barrier)
     }
     if (live)
     {
 #pragma unroll
-        for (int d = 0; d < DMAX; ++d)
-            if (d < D)
-                sp[(int64_t) d * V] = S[d];
+        for (int j = 0; j < DSZ; ++j)
+            if (d0 + j < D)
+                sp[(int64_t) (d0 + j) * V] = S[j];
     }
 }
 
@@ -519,9 +573,9 @@ int launch_stack_group_rmsnorm(void* y1, void* y2, const float* x, const int32_t
         return -1;
     }
     if (dtype == DT_BF16)
-        hipLaunchKernelGGL((group_rmsnorm_kernel<DT_BF16>), dim3(n_rows), dim3(256), 0, stream, y1, y2, x, rows, w1, w2, width, groups, eps);
+        hipLaunchKernelGGL((group_rmsnorm_kernel<DT_BF16>), dim3(n_rows, groups), dim3(GN_T), 0, stream, y1, y2, x, rows, w1, w2, width, groups, eps);
     else
-        hipLaunchKernelGGL((group_rmsnorm_kernel<DT_FLOAT>), dim3(n_rows), dim3(256), 0, stream, y1, y2, x, rows, w1, w2, width, groups, eps);
+        hipLaunchKernelGGL((group_rmsnorm_kernel<DT_FLOAT>), dim3(n_rows, groups), dim3(GN_T), 0, stream, y1, y2, x, rows, w1, w2, width, groups, eps);
     return launched("stack_group_rmsnorm");
 }
 
@@ -565,10 +619,13 @@ int launch_stack_rope_kv(const StackAttnParams& p, hipStream_t stream)
         return 0;
     if (!attn_shape_ok(p, "stack_rope_kv"))
         return -1;
+    // few rows (decoding): one element per thread; many rows: a workgroup per row walks it
+    const int per_row = (p.heads + p.kv_heads) * p.maps * p.dim;
+    const dim3 grid(p.tokens, p.tokens >= 64 ? 1 : (per_row + 255) / 256);
     if (p.dtype == DT_BF16)
-        hipLaunchKernelGGL((rope_kv_kernel<DT_BF16>), dim3(p.tokens), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((rope_kv_kernel<DT_BF16>), grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL((rope_kv_kernel<DT_FLOAT>), dim3(p.tokens), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((rope_kv_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, p);
     return launched("stack_rope_kv");
 }
 
@@ -644,36 +701,34 @@ int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
     }
     if (p.vdim <= 256)
     {
-        const dim3 hg(p.entries, p.heads);
-#define TLLM_HGRN_H(DT, DMAX)                                                                                                   \
+        // vpad x DS threads, DSZ state rows each: as many slices as fit 1024 threads, at least 8 rows per thread
+        const int vpad = (p.vdim + 63) / 64 * 64;
+        int DS = std::min(1024 / vpad, (p.dim + 7) / 8);
+        int dsz = (p.dim + DS - 1) / DS;
+        dsz = dsz <= 8 ? 8 : (dsz <= 16 ? 16 : 32);
+        DS = (p.dim + dsz - 1) / dsz;
+        const int NT = vpad * DS;
+        if (dsz * DS >= p.dim && NT <= 1024 && HTC * p.dim <= H_PPT * NT)
+        {
+            const size_t lds = sizeof(float) * ((size_t) 2 * HTC * p.dim + (size_t) HTC * vpad + (size_t) HTC * DS * vpad + (size_t) HTC * (vpad / 64));
+            const dim3 hg(p.entries, p.heads);
+#define TLLM_HGRN_H(DT)                                                                                                         \
     do                                                                                                                              \
     {                                                                                                                               \
-        if (p.vdim <= 64)                                                                                                           \
-            hipLaunchKernelGGL((hgrn2_head_kernel<DT, DMAX, 64>), hg, dim3(64), 0, stream, p);                                      \
-        else if (p.vdim <= 128)                                                                                                     \
-            hipLaunchKernelGGL((hgrn2_head_kernel<DT, DMAX, 128>), hg, dim3(128), 0, stream, p);                                    \
+        if (dsz == 8)                                                                                                               \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 8>), hg, dim3(NT), lds, stream, p, vpad, DS);                                 \
+        else if (dsz == 16)                                                                                                         \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 16>), hg, dim3(NT), lds, stream, p, vpad, DS);                                \
         else                                                                                                                        \
-            hipLaunchKernelGGL((hgrn2_head_kernel<DT, DMAX, 256>), hg, dim3(256), 0, stream, p);                                    \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 32>), hg, dim3(NT), lds, stream, p, vpad, DS);                                \
     } while (0)
-#define TLLM_HGRN_HD(DT)                                                                                                        \
-    do                                                                                                                              \
-    {                                                                                                                               \
-        if (p.dim <= 16)                                                                                                            \
-            TLLM_HGRN_H(DT, 16);                                                                                                    \
-        else if (p.dim <= 32)                                                                                                       \
-            TLLM_HGRN_H(DT, 32);                                                                                                    \
-        else if (p.dim <= 64)                                                                                                       \
-            TLLM_HGRN_H(DT, 64);                                                                                                    \
-        else                                                                                                                        \
-            TLLM_HGRN_H(DT, 128);                                                                                                   \
-    } while (0)
-        if (p.dtype == DT_BF16)
-            TLLM_HGRN_HD(DT_BF16);
-        else
-            TLLM_HGRN_HD(DT_FLOAT);
-#undef TLLM_HGRN_HD
+            if (p.dtype == DT_BF16)
+                TLLM_HGRN_H(DT_BF16);
+            else
+                TLLM_HGRN_H(DT_FLOAT);
 #undef TLLM_HGRN_H
-        return launched("stack_hgrn2 (head-wide)");
+            return launched("stack_hgrn2 (head-wide)");
+        }
     }
     const dim3 grid(p.entries, p.heads, (p.vdim + 63) / 64);
 #define TLLM_HGRN(DT, DMAX) hipLaunchKernelGGL((hgrn2_scan_kernel<DT, DMAX>), grid, dim3(64), 0, stream, p)
