@@ -57,6 +57,10 @@ MECHANISMS = {
     'hgrn2_alone_no_ff': make_config([hgrn2_layer()]),
     'hgrn2_small_heads': make_config([hgrn2_layer(heads=4, dim=8, vdim=8, ff=48)], groups=2),
     'hgrn2_wide': make_config([hgrn2_layer(heads=1, dim=72, vdim=136)]),
+    'hgrn2_wider_than_a_workgroup': make_config([hgrn2_layer(heads=1, dim=40, vdim=320)]),
+    'hgrn2_long_keys': make_config([hgrn2_layer(heads=2, dim=200, vdim=48)]),
+    'rows_that_are_not_16_byte_multiples': make_config([attention_layer(heads=3, kv_heads=1, dim=10, vdim=14, rot_dims=6, ff=50), hgrn2_layer(heads=3, dim=6, vdim=10, ff=34)],
+                                                       width=76, vocab=131, groups=19),
     'loop_three_passes': make_config(FULL[:3], loop=(0, 2, 3)),
     'loop_one_pass': make_config(FULL[:3], loop=(1, 3, 1)),
     'loop_whole_stack': make_config(FULL[:2], loop=(0, 2, 2), emb_scale=1.0),

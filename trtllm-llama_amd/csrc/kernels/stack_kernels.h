@@ -127,6 +127,7 @@ struct StackHgrnParams
     void* out = nullptr;           // [tokens, heads * vdim]
 };
 int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream);
+bool stack_hgrn2_serves(int32_t dim, int32_t vdim); // shapes one of its two forms takes
 
 } // namespace kernels
 } // namespace tllm

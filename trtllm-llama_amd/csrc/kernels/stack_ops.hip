@@ -687,16 +687,26 @@ float stack_rope_freqs(float* freq, int32_t dims, double base, double factor, do
     return factor > 0 ? (float) (0.1 * std::log(factor) + 1.0) : 1.f;
 }
 
+bool stack_hgrn2_serves(int32_t dim, int32_t vdim)
+{
+    if (dim < 1 || vdim < 1)
+        return false;
+    if (dim <= 128)
+        return true; // the column-per-thread form takes any vdim
+    const int vpad = (vdim + 63) / 64 * 64;
+    return vdim <= 256 && dim <= 32 * (1024 / vpad);
+}
+
 int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
 {
     if (p.tokens <= 0 || p.entries <= 0)
         return 0;
     if (!known_dtype(p.dtype, "stack_hgrn2"))
         return -1;
-    if (p.heads < 1 || p.dim < 1 || p.vdim < 1 || p.dim > 128)
+    if (p.heads < 1 || !stack_hgrn2_serves(p.dim, p.vdim))
     {
-        set_error("stack_hgrn2: heads %d, dim %d, vdim %d is not a shape it serves (dim <= 128: a state column lives in registers)", p.heads,
-            p.dim, p.vdim);
+        set_error("stack_hgrn2: heads %d, dim %d, vdim %d is not a shape it serves (a thread keeps up to 32 state rows of a column: dim <= 128, or "
+                  "vdim <= 256 and dim <= 32 * (1024 / vdim rounded up to 64))", p.heads, p.dim, p.vdim);
         return -1;
     }
     if (p.vdim <= 256)
@@ -729,6 +739,11 @@ int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
 #undef TLLM_HGRN_H
             return launched("stack_hgrn2 (head-wide)");
         }
+    }
+    if (p.dim > 128)
+    {
+        set_error("stack_hgrn2: dim %d with vdim %d fits neither form", p.dim, p.vdim);
+        return -1;
     }
     const dim3 grid(p.entries, p.heads, (p.vdim + 63) / 64);
 #define TLLM_HGRN(DT, DMAX) hipLaunchKernelGGL((hgrn2_scan_kernel<DT, DMAX>), grid, dim3(64), 0, stream, p)

@@ -367,8 +367,8 @@ tllm_stack_t tllm_stack_create(const char* config_text)
         }
         else
         {
-            if (l.dim > 128)
-                return fail("hgrn2: dim up to 128");
+            if (!stack_hgrn2_serves(l.dim, l.vdim))
+                return fail("hgrn2: dim up to 128, or vdim up to 256 with dim up to 32 * (1024 / vdim rounded up to 64)");
             l.n_q = l.heads * l.dim;
             l.n_k = l.heads * l.dim; // forget gate
             l.n_v = l.heads * l.vdim;
