@@ -12,6 +12,7 @@
 #include "dev_utils.h"
 #include "launch_util.h"
 #include "stack_kernels.h"
+#include <algorithm>
 #include <cstdlib>
 
 namespace tllm
@@ -24,6 +25,7 @@ using namespace dev;
 
 namespace
 {
+constexpr int kSplitRows = 64, kMaxSplits = 16;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -109,13 +111,17 @@ __device__ __forceinline__ uint4 softmax_block(f32x4 (&s)[2], float& m_run, floa
 }
 
 template <int MAPS, int DK, int VT, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParams p, int below_count)
+__global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParams p, int below_count, int ks)
 {
     constexpr int D = DK * 32, V = VT * 16;
     extern __shared__ float lds[];
     float* o_part = lds;                          // [NW][MAPS][16][V]
     float* ml_part = lds + NW * MAPS * 16 * V;    // [NW][MAPS][16][2]
-    const int e = blockIdx.y, h = blockIdx.z, r0 = blockIdx.x * 16;
+    // ks == 1: blockIdx.x is the entry's 16-row tile.  ks > 1 (decoding steps: every entry one tile): blockIdx.x is the key split -
+    // workgroup `split` of an (entry, head) takes the key blocks split * NW + w, + ks * NW, ... and leaves an unnormalised partial
+    // (max, sum, O per map and row) in split_ws; attn_split_merge_kernel finishes the rows.
+    const int e = blockIdx.y, h = blockIdx.z, r0 = ks > 1 ? 0 : blockIdx.x * 16;
+    const int split = ks > 1 ? blockIdx.x : 0;
     const int count = p.ent_count[e];
     if (r0 >= count || count >= below_count) // entries of below_count rows and more are the prefill form's
         return;
@@ -171,10 +177,11 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
                     kf[m][t][ks] = *reinterpret_cast<const uint4*>(krow + ks * 32);
             }
     };
-    int blk = w < nblk ? table[w * 32 / page] : 0;
-    if (w < nblk)
-        request_k(w, blk);
-    for (int kb = w; kb < nblk; kb += NW)
+    const int kb0 = split * NW + w, kstep = ks * NW;
+    int blk = kb0 < nblk ? table[kb0 * 32 / page] : 0;
+    if (kb0 < nblk)
+        request_k(kb0, blk);
+    for (int kb = kb0; kb < nblk; kb += kstep)
     {
         const int key0 = kb * 32, off = key0 % page;
         uint2 vlo[VT], vhi[VT];
@@ -198,10 +205,10 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
                 for (int ks = 0; ks < DK; ++ks)
                     s[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[m][t][ks]), qf[m][ks], s[m][t], 0, 0, 0);
             }
-        if (kb + NW < nblk)
+        if (kb + kstep < nblk)
         {
-            blk = table[(key0 + NW * 32) / page];
-            request_k(kb + NW, blk);
+            blk = table[(key0 + kstep * 32) / page];
+            request_k(kb + kstep, blk);
         }
         uint4 pf[MAPS]; // P^T fragment of the block, 8 bfloat16 per map
         const bool masked = key0 + 31 > pos0 + r0; // wave-uniform
@@ -254,11 +261,49 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
             wgt[m][ww] = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M); // the running maxima are base-2 exponents
             L += wgt[m][ww] * ml_part[((ww * MAPS + m) * 16 + row) * 2 + 1];
         }
+        if (ks > 1)
+        {
+            // partial of this split: weights stay relative to the split's own maximum, nothing is divided yet
+            if (sub == 0 && r0 + row < count)
+            {
+                float* ws = p.split_ws + ((((int64_t) (first + row) * p.heads + h) * ks + split) * MAPS + m) * (V + 2);
+                ws[V] = M;
+                ws[V + 1] = L;
+            }
+        }
+        else
+        {
 #pragma unroll
-        for (int ww = 0; ww < NW; ++ww)
-            wgt[m][ww] /= L;
+            for (int ww = 0; ww < NW; ++ww)
+                wgt[m][ww] /= L;
+        }
     }
     constexpr int CPT = (V + TPR - 1) / TPR;
+    if (ks > 1)
+    {
+        if (r0 + row < count)
+        {
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m)
+            {
+                float* ws = p.split_ws + ((((int64_t) (first + row) * p.heads + h) * ks + split) * MAPS + m) * (V + 2);
+#pragma unroll
+                for (int c = 0; c < CPT; ++c)
+                {
+                    const int ch = sub + c * TPR;
+                    if (ch < V)
+                    {
+                        float a = 0.f;
+#pragma unroll
+                        for (int ww = 0; ww < NW; ++ww)
+                            a += wgt[m][ww] * o_part[((ww * MAPS + m) * 16 + row) * V + ch];
+                        ws[ch] = a;
+                    }
+                }
+            }
+        }
+        return;
+    }
     float o[CPT], ss = 0.f;
 #pragma unroll
     for (int c = 0; c < CPT; ++c)
@@ -476,6 +521,71 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
     }
 }
 
+// Second pass of the key split: one wave per (row, head) combines the ks partials of each map, then the differential combination,
+// the head norm and the bfloat16 store.
+template <int MAPS>
+__global__ __launch_bounds__(64) void attn_split_merge_kernel(const StackAttnParams p, int ks, int below_count)
+{
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    if (p.ent_count[p.tok_entry[t]] >= below_count)
+        return;
+    const int V = p.vdim;
+    const float* base = p.split_ws + (((int64_t) t * p.heads + h) * ks) * MAPS * (V + 2);
+    // lane l < ks * MAPS owns partial (split l / MAPS, map l % MAPS): all maxima and sums are fetched at once, the weights are
+    // formed with wave reductions and handed to the channel lanes by shuffles
+    const bool owner = lane < ks * MAPS;
+    const float pm = owner ? base[lane * (V + 2) + V] : -INFINITY;
+    const float pl = owner ? base[lane * (V + 2) + V + 1] : 0.f;
+    float wl = 0.f;
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+    {
+        const bool mine = owner && lane % MAPS == m;
+        const float M = wave_max(mine ? pm : -INFINITY);
+        const float e_ = mine && pm != -INFINITY ? __builtin_amdgcn_exp2f(pm - M) : 0.f;
+        const float L = wave_sum(e_ * pl);
+        if (mine)
+            wl = e_ / L;
+    }
+    float o[2], ss = 0.f; // vdim <= 128: two channels per lane
+    float a[2][MAPS];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m)
+            a[c][m] = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxSplits * MAPS; ++i)
+    {
+        const float wgt = __shfl(wl, i, 64);
+        if (i < ks * MAPS) // wave-uniform
+        {
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+                if (lane + c * 64 < V)
+                    a[c][i % MAPS] += wgt * base[i * (V + 2) + lane + c * 64];
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+    {
+        o[c] = 0.f;
+        if (lane + c * 64 < V)
+        {
+            o[c] = MAPS == 2 ? a[c][0] - p.lambda * a[c][MAPS - 1] : a[c][0];
+            ss += o[c] * o[c];
+        }
+    }
+    float mul = 1.f;
+    if (p.head_norm)
+        mul = p.out_scale / sqrtf(wave_sum(ss) / (float) V + p.eps);
+    uint16_t* out = reinterpret_cast<uint16_t*>(p.out) + ((int64_t) t * p.heads + h) * V;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+        if (lane + c * 64 < V)
+            out[lane + c * 64] = f2bf(o[c] * mul);
+}
+
 template <int MAPS, int DK, int VT>
 int launch_tile(const StackAttnParams& p, hipStream_t stream)
 {
@@ -497,8 +607,18 @@ int launch_tile(const StackAttnParams& p, hipStream_t stream)
     }
     if (small_rows > 0)
     {
-        const dim3 grid((small_rows + 15) / 16, p.entries, p.heads);
-        hipLaunchKernelGGL((attn_tile_kernel<MAPS, DK, VT, NW>), grid, dim3(NW * 64), lds, stream, p, PREFILL_ROWS);
+        // a step of decoded tokens only (every entry within one tile, few rows in all): the keys of an (entry, head) are split over
+        // ks workgroups so that a long context is walked by ks * NW waves, two key blocks or so each
+        int ks = 1;
+        if (p.split_ws && p.max_count <= 16 && p.tokens <= kSplitRows)
+        {
+            const int nblk = (p.max_context + 31) / 32;
+            ks = std::min(kMaxSplits, (nblk + 2 * NW - 1) / (2 * NW));
+        }
+        const dim3 grid(ks > 1 ? ks : (small_rows + 15) / 16, p.entries, p.heads);
+        hipLaunchKernelGGL((attn_tile_kernel<MAPS, DK, VT, NW>), grid, dim3(NW * 64), lds, stream, p, PREFILL_ROWS, ks);
+        if (ks > 1)
+            hipLaunchKernelGGL((attn_split_merge_kernel<MAPS>), dim3(p.tokens, p.heads), dim3(64), 0, stream, p, ks, PREFILL_ROWS);
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess)
@@ -535,9 +655,10 @@ int launch_tile_d(const StackAttnParams& p, hipStream_t stream)
 
 } // namespace
 
-size_t stack_attn_workspace_floats(int32_t tokens, int32_t heads, int32_t maps, int32_t vdim)
+// partials of the cross-workgroup key split: steps of up to kSplitRows rows, up to kMaxSplits splits per (row, head)
+size_t stack_attn_workspace_floats(int32_t heads, int32_t maps, int32_t vdim)
 {
-    return 0; // the key-split waves of a workgroup merge through LDS
+    return (size_t) kSplitRows * heads * kMaxSplits * maps * (vdim + 2);
 }
 
 // the tile kernel's shapes: bfloat16, dim 32 / 64 / 128, vdim 32 / 64 / 128, pages of a multiple of 32 keys

@@ -92,13 +92,13 @@ struct StackAttnParams
     int32_t max_count = 0;                // host: the largest ent_count of the step
     int32_t max_context = 0;              // host: the largest pos0 + count of the step
     void* out = nullptr;                  // [tokens, heads * vdim]
-    float* split_ws = nullptr;            // decode: partials of the key splits (stack_attn_workspace_floats)
+    float* split_ws = nullptr;            // decoding steps: partials of the cross-workgroup key split (stack_attn_workspace_floats); null: no split
 };
 // rotates q and k, appends k and v of the step's rows to the paged cache
 int launch_stack_rope_kv(const StackAttnParams& p, hipStream_t stream);
 // causal attention of the step's rows over their sequences' cache (which already holds the step's own keys)
 int launch_stack_attention(const StackAttnParams& p, hipStream_t stream);
-size_t stack_attn_workspace_floats(int32_t tokens, int32_t heads, int32_t maps, int32_t vdim);
+size_t stack_attn_workspace_floats(int32_t heads, int32_t maps, int32_t vdim); // floats of split_ws a layer of this shape needs
 // frequencies of the rotation with YaRN-style scaling (factor <= 0: none): fills freq[dims / 2], returns the cos / sin multiplier
 float stack_rope_freqs(float* freq, int32_t dims, double base, double factor, double original, double fast, double slow);
 

@@ -79,7 +79,7 @@ struct tllm_stack
     std::vector<Layer> layers;
     std::vector<Run> runs;
     void *embed = nullptr, *head = nullptr;
-    float *final_norm = nullptr, *loop_step = nullptr;
+    float *final_norm = nullptr, *loop_step = nullptr, *attn_ws = nullptr;
     bool finalized = false;
     int64_t weight_bytes = 0;
     std::vector<void*> owned;
@@ -516,6 +516,17 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
                 return -1;
         }
     }
+    size_t ws_floats = 0;
+    for (const Layer& l : s->layers)
+        if (l.kind == MIX_ATTENTION)
+            ws_floats = std::max(ws_floats, stack_attn_workspace_floats(l.heads, l.maps, l.vdim));
+    if (ws_floats)
+    {
+        void* ws = nullptr;
+        if (alloc_zero(s, ws_floats * 4, &ws))
+            return -1;
+        s->attn_ws = (float*) ws;
+    }
     for (Run& r : s->runs)
     {
         const Layer& l = s->layers[r.layer];
@@ -700,6 +711,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
             a.max_count = max_count;
             a.max_context = max_ctx;
             a.out = s->ctx;
+            a.split_ws = s->attn_ws;
             if (launch_stack_rope_kv(a, stream) || launch_stack_attention(a, stream))
                 return -1;
         }
