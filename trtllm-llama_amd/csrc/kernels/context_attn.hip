@@ -530,7 +530,7 @@ __global__ __launch_bounds__(128 * NQ) void context_attn_mfma_ks_kernel(const Co
     // The Q fragments are consumed here, in front of the first LDS-DMA: hipcc does not see the hand-written vmcnt wait at the top of
     // the loop, so it kept its own `s_waitcnt vmcnt(7) .. vmcnt(0)` for these eight loads in front of the eight QK MFMAs of EVERY
     // iteration - where the only memory operations still in flight are this wave's LDS-DMA pieces of the NEXT block, which the
-    // last MFMA of the block then waited for (r02, found in the ISA: the DMA latency sat inside the compute chain of every step).
+    // last MFMA of the block then waited for: the DMA latency sat inside the compute chain of every step.
 #pragma unroll
     for (int s = 0; s < KST; ++s)
         asm volatile("" : "+v"(qf[s].x), "+v"(qf[s].y), "+v"(qf[s].z), "+v"(qf[s].w));
