@@ -582,10 +582,10 @@ def tolenex_config(width, layers, vocab=32000):
     128 x 128 states, feed-forward 2.6875 x width."""
     heads = width // 128
     attn = {'type': 'attention', 'mlp': {'ff': int(width * 2.6875), 'kind': 'dense'},
-            'mixer': {'heads': heads, 'kv_heads': max(heads // 4, 1), 'dim': 64, 'vdim': 128, 'diff': 0.3, 'scale': 0.125, 'softcap': 50.0,
-                      'rot': {'dims': 64, 'base': 1000000.0, 'scaling': {'factor': 8.0, 'original': 4096, 'fast': 32.0, 'slow': 1.0}}}}
+            'mixer': {'heads': heads, 'kv_heads': max(heads // 4, 1), 'dim': 64, 'vdim': 128, 'diff': 0.2, 'scale': 0.125, 'softcap': 30.0,
+                      'rot': {'dims': 64, 'base': 500000.0, 'scaling': {'factor': 4.0, 'original': 8192, 'fast': 16.0, 'slow': 2.0}}}}
     rec = {'type': 'hgrn2', 'mlp': {'ff': int(width * 2.6875), 'kind': 'dense'}, 'mixer': {'heads': heads, 'dim': 128, 'vdim': 128}}
-    return {'architecture': 'Tolenex', 'vocab': vocab, 'width': width, 'embedding': {'scale': 8.0}, 'norm': {'eps': 1e-5, 'groups': 2},
+    return {'architecture': 'Tolenex', 'vocab': vocab, 'width': width, 'embedding': {'scale': 8.0}, 'norm': {'eps': 1e-6, 'groups': 4},
             'layers': [rec if i % 4 == 2 else attn for i in range(layers)]}
 
 
