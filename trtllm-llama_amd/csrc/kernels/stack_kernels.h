@@ -123,6 +123,7 @@ struct StackHgrnParams
     const int32_t* ent_first = nullptr;
     const int32_t* ent_count = nullptr;
     const int32_t* ent_pos0 = nullptr;
+    int32_t max_count = 0;         // host: the largest ent_count of the step
     float* o32 = nullptr;          // scratch [tokens, heads * vdim]
     void* out = nullptr;           // [tokens, heads * vdim]
 };

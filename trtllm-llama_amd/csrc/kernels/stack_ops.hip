@@ -397,7 +397,7 @@ __global__ __launch_bounds__(64) void hgrn2_scan_kernel(const StackHgrnParams p)
 constexpr int HTC = 8, H_PPT = 4;
 
 template <int DT, int DSZ>
-__global__ __launch_bounds__(1024) void hgrn2_head_kernel(const StackHgrnParams p, int vpad, int DS)
+__global__ __launch_bounds__(1024) void hgrn2_head_kernel(const StackHgrnParams p, int vpad, int DS, int fuse_norm)
 {
     extern __shared__ float hsm[];
     const int D = p.dim, V = p.vdim, HD = p.heads * D, NT = blockDim.x;
@@ -406,7 +406,9 @@ __global__ __launch_bounds__(1024) void hgrn2_head_kernel(const StackHgrnParams 
     float* os = vs + HTC * vpad;                        // [HTC][DS][vpad]
     float* red = os + HTC * DS * vpad;                  // [HTC][vpad / 64]
     const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-    const int s = tid / vpad, v = tid % vpad, lane = tid & 63, vw = v >> 6, nvw = vpad >> 6;
+    // the workgroup's columns: [blockIdx.z * vpad, + vpad).  fuse_norm: one workgroup holds the whole head (vpad a multiple of 64, a
+    // wave one slice) and norms it; otherwise a head is spread over several workgroups, o goes out in fp32 and a pass norms it
+    const int s = tid / vpad, vl = tid % vpad, v = blockIdx.z * vpad + vl, lane = tid & 63, vw = vl >> 6, nvw = (vpad + 63) >> 6;
     const int first = p.ent_first[e], count = p.ent_count[e];
     const bool live = v < V;
     const int d0 = s * DSZ;
@@ -418,26 +420,30 @@ __global__ __launch_bounds__(1024) void hgrn2_head_kernel(const StackHgrnParams 
         S[j] = (live && d0 + j < D && carry) ? sp[(int64_t) (d0 + j) * V] : 0.f;
     const float nw = live ? p.norm_w[v] : 0.f;
 
-    float rq[H_PPT], rf[H_PPT], rv[HTC];
-    auto request = [&](int t0) {
+    // raw projections of the next chunk (rq / rf / rv) and of the one behind it (nq / nf / nv): a chunk's loads are issued two
+    // chunks before it is computed, so a chunk waits for memory only at the very start of an entry
+    float rq[H_PPT], rf[H_PPT], rv[HTC], nq[H_PPT], nf[H_PPT], nv[HTC];
+    auto request = [&](int t0, float (&q_)[H_PPT], float (&f_)[H_PPT], float (&v_)[HTC]) {
         const int nt = count - t0 < HTC ? count - t0 : HTC;
 #pragma unroll
         for (int k = 0; k < H_PPT; ++k)
         {
             const int i = tid + k * NT;
-            rq[k] = rf[k] = 0.f;
+            q_[k] = f_[k] = 0.f;
             if (i < nt * D)
             {
                 const int64_t row = (int64_t) (first + t0 + i / D) * p.ldp;
-                rq[k] = El<DT>::ld(p.proj, row + h * D + i % D);
-                rf[k] = El<DT>::ld(p.proj, row + HD + h * D + i % D);
+                q_[k] = El<DT>::ld(p.proj, row + h * D + i % D);
+                f_[k] = El<DT>::ld(p.proj, row + HD + h * D + i % D);
             }
         }
 #pragma unroll
         for (int tt = 0; tt < HTC; ++tt)
-            rv[tt] = (s == 0 && live && tt < nt) ? El<DT>::ld(p.proj, (int64_t) (first + t0 + tt) * p.ldp + 2 * HD + h * V + v) : 0.f;
+            v_[tt] = (s == 0 && live && tt < nt) ? El<DT>::ld(p.proj, (int64_t) (first + t0 + tt) * p.ldp + 2 * HD + h * V + v) : 0.f;
     };
-    request(0);
+    request(0, rq, rf, rv);
+    if (HTC < count)
+        request(HTC, nq, nf, nv);
     for (int t0 = 0; t0 < count; t0 += HTC)
     {
         const int nt = count - t0 < HTC ? count - t0 : HTC;
@@ -459,14 +465,26 @@ __global__ __launch_bounds__(1024) void hgrn2_head_kernel(const StackHgrnParams 
         {
 #pragma unroll
             for (int tt = 0; tt < HTC; ++tt)
-                vs[tt * vpad + v] = rv[tt];
+                vs[tt * vpad + vl] = rv[tt];
         }
         __syncthreads();
         if (t0 + HTC < count)
-            request(t0 + HTC); // in flight under the recurrence
+        {
+#pragma unroll
+            for (int k = 0; k < H_PPT; ++k)
+            {
+                rq[k] = nq[k];
+                rf[k] = nf[k];
+            }
+#pragma unroll
+            for (int tt = 0; tt < HTC; ++tt)
+                rv[tt] = nv[tt];
+            if (t0 + 2 * HTC < count)
+                request(t0 + 2 * HTC, nq, nf, nv); // in flight under this chunk's and the next chunk's recurrence
+        }
         for (int tt = 0; tt < nt; ++tt)
         {
-            const float x = vs[tt * vpad + v];
+            const float x = vs[tt * vpad + vl];
             float o = 0.f;
 #pragma unroll
             for (int j = 0; j < DSZ; ++j)
@@ -478,15 +496,30 @@ __global__ __launch_bounds__(1024) void hgrn2_head_kernel(const StackHgrnParams 
                     o += S[j] * c.y;
                 }
             }
-            os[(tt * DS + s) * vpad + v] = live ? o : 0.f;
+            os[(tt * DS + s) * vpad + vl] = live ? o : 0.f;
         }
         __syncthreads();
         // rows of the chunk are shared out over the slices: thread (s, v) finishes rows s, s + DS, ...
+        if (!fuse_norm)
+        {
+            for (int tt = s; tt < nt; tt += DS)
+            {
+                if (live)
+                {
+                    float o = 0.f;
+                    for (int s2 = 0; s2 < DS; ++s2)
+                        o += os[(tt * DS + s2) * vpad + vl];
+                    p.o32[(int64_t) (first + t0 + tt) * (p.heads * V) + h * V + v] = o;
+                }
+            }
+            __syncthreads();
+            continue;
+        }
         for (int tt = s; tt < nt; tt += DS) // wave-uniform
         {
             float o = 0.f;
             for (int s2 = 0; s2 < DS; ++s2)
-                o += os[(tt * DS + s2) * vpad + v];
+                o += os[(tt * DS + s2) * vpad + vl];
             const float ss = wave_sum(o * o);
             if (lane == 0)
                 red[tt * nvw + vw] = ss;
@@ -498,7 +531,7 @@ __global__ __launch_bounds__(1024) void hgrn2_head_kernel(const StackHgrnParams 
             {
                 float o = 0.f, ss = 0.f;
                 for (int s2 = 0; s2 < DS; ++s2)
-                    o += os[(tt * DS + s2) * vpad + v];
+                    o += os[(tt * DS + s2) * vpad + vl];
                 for (int w = 0; w < nvw; ++w)
                     ss += red[tt * nvw + w];
                 El<DT>::st(p.out, (int64_t) (first + t0 + tt) * (p.heads * V) + h * V + v, o * (1.f / sqrtf(ss / (float) V + p.eps)) * nw);
@@ -691,10 +724,7 @@ bool stack_hgrn2_serves(int32_t dim, int32_t vdim)
 {
     if (dim < 1 || vdim < 1)
         return false;
-    if (dim <= 128)
-        return true; // the column-per-thread form takes any vdim
-    const int vpad = (vdim + 63) / 64 * 64;
-    return vdim <= 256 && dim <= 32 * (1024 / vpad);
+    return dim <= 2048; // 16-column groups x 64 slices of 32 rows; up to 128 the column-per-thread form serves too
 }
 
 int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
@@ -705,39 +735,62 @@ int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
         return -1;
     if (p.heads < 1 || !stack_hgrn2_serves(p.dim, p.vdim))
     {
-        set_error("stack_hgrn2: heads %d, dim %d, vdim %d is not a shape it serves (a thread keeps up to 32 state rows of a column: dim <= 128, or "
-                  "vdim <= 256 and dim <= 32 * (1024 / vdim rounded up to 64))", p.heads, p.dim, p.vdim);
+        set_error("stack_hgrn2: heads %d, dim %d, vdim %d is not a shape it serves (dim up to 2048)", p.heads, p.dim, p.vdim);
         return -1;
     }
-    if (p.vdim <= 256)
     {
-        // vpad x DS threads, DSZ state rows each: as many slices as fit 1024 threads, at least 8 rows per thread
-        const int vpad = (p.vdim + 63) / 64 * 64;
-        int DS = std::min(1024 / vpad, (p.dim + 7) / 8);
-        int dsz = (p.dim + DS - 1) / DS;
-        dsz = dsz <= 8 ? 8 : (dsz <= 16 ? 16 : 32);
-        DS = (p.dim + dsz - 1) / dsz;
-        const int NT = vpad * DS;
-        if (dsz * DS >= p.dim && NT <= 1024 && HTC * p.dim <= H_PPT * NT)
+        // Long portions (a prompt): a head is cut into groups of 16 columns, one workgroup each, so that the sequential walk over
+        // the rows runs on many CUs at once; the head norm is then a pass of its own.  Short portions and decoded tokens: one
+        // workgroup holds the whole head (vdim <= 256) and norms it in the same launch.
+        bool spread = p.max_count >= 32 || p.vdim > 256;
+        int vpad = 0, DS = 0, dsz = 0, NT = 0;
+        auto shape = [&]() {
+            vpad = spread ? 16 : (p.vdim + 63) / 64 * 64;
+            DS = std::min(1024 / vpad, (p.dim + 7) / 8);
+            dsz = (p.dim + DS - 1) / DS;
+            dsz = dsz <= 8 ? 8 : (dsz <= 16 ? 16 : 32);
+            DS = (p.dim + dsz - 1) / dsz;
+            NT = vpad * DS;
+            return dsz * DS >= p.dim && NT <= 1024 && HTC * p.dim <= H_PPT * NT;
+        };
+        bool fits = shape();
+        if (!fits && !spread)
         {
-            const size_t lds = sizeof(float) * ((size_t) 2 * HTC * p.dim + (size_t) HTC * vpad + (size_t) HTC * DS * vpad + (size_t) HTC * (vpad / 64));
-            const dim3 hg(p.entries, p.heads);
+            spread = true; // a head too tall for one workgroup: the column groups take it
+            fits = shape();
+        }
+        if (fits)
+        {
+            const size_t lds = sizeof(float) * ((size_t) 2 * HTC * p.dim + (size_t) HTC * vpad + (size_t) HTC * DS * vpad + (size_t) HTC * ((vpad + 63) / 64));
+            const dim3 hg(p.entries, p.heads, spread ? (p.vdim + vpad - 1) / vpad : 1);
+            const int fuse = spread ? 0 : 1;
 #define TLLM_HGRN_H(DT)                                                                                                         \
     do                                                                                                                              \
     {                                                                                                                               \
         if (dsz == 8)                                                                                                               \
-            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 8>), hg, dim3(NT), lds, stream, p, vpad, DS);                                 \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 8>), hg, dim3(NT), lds, stream, p, vpad, DS, fuse);                           \
         else if (dsz == 16)                                                                                                         \
-            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 16>), hg, dim3(NT), lds, stream, p, vpad, DS);                                \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 16>), hg, dim3(NT), lds, stream, p, vpad, DS, fuse);                          \
         else                                                                                                                        \
-            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 32>), hg, dim3(NT), lds, stream, p, vpad, DS);                                \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 32>), hg, dim3(NT), lds, stream, p, vpad, DS, fuse);                          \
     } while (0)
             if (p.dtype == DT_BF16)
                 TLLM_HGRN_H(DT_BF16);
             else
                 TLLM_HGRN_H(DT_FLOAT);
 #undef TLLM_HGRN_H
-            return launched("stack_hgrn2 (head-wide)");
+            if (launched("stack_hgrn2 (sliced)"))
+                return -1;
+            if (fuse)
+                return 0;
+            const int64_t nh = (int64_t) p.tokens * p.heads;
+            if (p.dtype == DT_BF16)
+                hipLaunchKernelGGL((head_rmsnorm_kernel<DT_BF16>), dim3((unsigned) ((nh + 3) / 4)), dim3(256), 0, stream, p.out, p.o32, p.norm_w,
+                    nh, p.vdim, p.eps);
+            else
+                hipLaunchKernelGGL((head_rmsnorm_kernel<DT_FLOAT>), dim3((unsigned) ((nh + 3) / 4)), dim3(256), 0, stream, p.out, p.o32, p.norm_w,
+                    nh, p.vdim, p.eps);
+            return launched("stack_hgrn2 norm");
         }
     }
     if (p.dim > 128)

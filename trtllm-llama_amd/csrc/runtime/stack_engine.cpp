@@ -368,7 +368,7 @@ tllm_stack_t tllm_stack_create(const char* config_text)
         else
         {
             if (!stack_hgrn2_serves(l.dim, l.vdim))
-                return fail("hgrn2: dim up to 128, or vdim up to 256 with dim up to 32 * (1024 / vdim rounded up to 64)");
+                return fail("hgrn2: dim up to 2048");
             l.n_q = l.heads * l.dim;
             l.n_k = l.heads * l.dim; // forget gate
             l.n_v = l.heads * l.vdim;
@@ -735,6 +735,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
             hp.ent_first = d_first;
             hp.ent_count = d_count;
             hp.ent_pos0 = d_pos0;
+            hp.max_count = max_count;
             hp.o32 = s->o32;
             hp.out = s->ctx;
             if (launch_stack_hgrn2(hp, stream))
