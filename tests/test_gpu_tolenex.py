@@ -134,6 +134,20 @@ def test_unequal_requests_in_one_batch_equal_each_alone(dtype, stack):
     assert not s.live() and s.cache.blocks_manager.num_free_blocks() == s.num_blocks and s.slots.num_free_slots() == 4
 
 
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+def test_requests_of_very_unequal_length_decode_side_by_side(dtype):
+    """Steps of decoded tokens only, one request far ahead of the others: the keys of the long one are walked by several
+    workgroups whose share of a short request is empty."""
+    cfg = make_config([TILED[0], TILED[2], hgrn2_layer(heads=2, dim=32, vdim=64, ff=40)], loop=(0, 2, 2))
+    w = random_weights(cfg, seed=21)
+    reqs = {'long': tokens_for(cfg, 620, 90), 'mid': tokens_for(cfg, 75, 91), 'new': tokens_for(cfg, 12, 92)}
+    schedule = [[('long', 600)], [('mid', 65), ('long', 1)]] + [[('long', 1), ('mid', 1), ('new', 1)]] * 10 + [[('long', 9), ('new', 2)]]
+    s = session_for(cfg, w, dtype, max_tokens=1024)
+    got = replay(s, reqs, schedule)
+    for rid, toks in reqs.items():
+        check(got[rid], O.tolenex_logits(toks, as_f64(w), cfg), F32_TOL if dtype == 'float32' else BF16_TOL, rid)
+
+
 def test_pages_and_slots_that_are_used_again():
     """A pool of 4 pages and 2 slots serves six requests one after another and side by side: every page and slot is written by
     several requests, and a recurrent state must start from zero in a slot another request has left."""
