@@ -394,10 +394,11 @@ __global__ __launch_bounds__(64) void hgrn2_scan_kernel(const StackHgrnParams p)
 // computed once per (row, channel of dim), its raw projections having been requested while the chunk before it was in the
 // recurrence; the recurrence itself has no cross-lane traffic, the DS partial outputs of a row meet in LDS once per chunk, and the
 // per-head RMS norm of the outputs is taken in the same launch (no fp32 round trip of o, no second kernel).
-constexpr int HTC = 8, H_PPT = 4;
+// HTC rows per chunk (8; 16 measured the same: the time goes with the rows, not with the chunks), H_PPT (row, channel) pairs of gate /
+// query work per thread and chunk: 4 where one workgroup of up to 1024 threads holds a head, DSZ / 2 in the 16-column groups of up to 256.
 
-template <int DT, int DSZ>
-__global__ __launch_bounds__(1024) void hgrn2_head_kernel(const StackHgrnParams p, int vpad, int DS, int fuse_norm)
+template <int DT, int DSZ, int HTC, int H_PPT, int MAXT>
+__global__ __launch_bounds__(MAXT) void hgrn2_head_kernel(const StackHgrnParams p, int vpad, int DS, int fuse_norm)
 {
     extern __shared__ float hsm[];
     const int D = p.dim, V = p.vdim, HD = p.heads * D, NT = blockDim.x;
@@ -724,7 +725,7 @@ bool stack_hgrn2_serves(int32_t dim, int32_t vdim)
 {
     if (dim < 1 || vdim < 1)
         return false;
-    return dim <= 2048; // 16-column groups x 64 slices of 32 rows; up to 128 the column-per-thread form serves too
+    return dim <= 512; // 16-column groups x 16 slices of 32 rows; up to 128 the column-per-thread form serves too
 }
 
 int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
@@ -735,7 +736,7 @@ int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
         return -1;
     if (p.heads < 1 || !stack_hgrn2_serves(p.dim, p.vdim))
     {
-        set_error("stack_hgrn2: heads %d, dim %d, vdim %d is not a shape it serves (dim up to 2048)", p.heads, p.dim, p.vdim);
+        set_error("stack_hgrn2: heads %d, dim %d, vdim %d is not a shape it serves (dim up to 512)", p.heads, p.dim, p.vdim);
         return -1;
     }
     {
@@ -743,15 +744,18 @@ int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
         // the rows runs on many CUs at once; the head norm is then a pass of its own.  Short portions and decoded tokens: one
         // workgroup holds the whole head (vdim <= 256) and norms it in the same launch.
         bool spread = p.max_count >= 32 || p.vdim > 256;
-        int vpad = 0, DS = 0, dsz = 0, NT = 0;
+        int vpad = 0, DS = 0, dsz = 0, NT = 0, htc = 0, ppt = 0;
         auto shape = [&]() {
             vpad = spread ? 16 : (p.vdim + 63) / 64 * 64;
-            DS = std::min(1024 / vpad, (p.dim + 7) / 8);
+            htc = 8;
+            const int max_threads = spread ? 256 : 1024;
+            DS = std::min(max_threads / vpad, (p.dim + 7) / 8);
             dsz = (p.dim + DS - 1) / DS;
             dsz = dsz <= 8 ? 8 : (dsz <= 16 ? 16 : 32);
             DS = (p.dim + dsz - 1) / dsz;
             NT = vpad * DS;
-            return dsz * DS >= p.dim && NT <= 1024 && HTC * p.dim <= H_PPT * NT;
+            ppt = spread ? dsz / 2 : 4; // (row, channel) pairs per thread and chunk: 8 * dim / NT <= dsz / 2 resp. 8 * dsz / vpad <= 4
+            return dsz * DS >= p.dim && NT <= max_threads && htc * p.dim <= ppt * NT;
         };
         bool fits = shape();
         if (!fits && !spread)
@@ -761,24 +765,33 @@ int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream)
         }
         if (fits)
         {
-            const size_t lds = sizeof(float) * ((size_t) 2 * HTC * p.dim + (size_t) HTC * vpad + (size_t) HTC * DS * vpad + (size_t) HTC * ((vpad + 63) / 64));
+            const size_t lds = sizeof(float) * ((size_t) 2 * htc * p.dim + (size_t) htc * vpad + (size_t) htc * DS * vpad + (size_t) htc * ((vpad + 63) / 64));
             const dim3 hg(p.entries, p.heads, spread ? (p.vdim + vpad - 1) / vpad : 1);
             const int fuse = spread ? 0 : 1;
+#define TLLM_HGRN_K(DT, DSZ)                                                                                                    \
+    do                                                                                                                              \
+    {                                                                                                                               \
+        if (spread)                                                                                                                 \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, DSZ, 8, DSZ / 2, 256>), hg, dim3(NT), lds, stream, p, vpad, DS, fuse);                  \
+        else                                                                                                                        \
+            hipLaunchKernelGGL((hgrn2_head_kernel<DT, DSZ, 8, 4, 1024>), hg, dim3(NT), lds, stream, p, vpad, DS, fuse);                   \
+    } while (0)
 #define TLLM_HGRN_H(DT)                                                                                                         \
     do                                                                                                                              \
     {                                                                                                                               \
         if (dsz == 8)                                                                                                               \
-            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 8>), hg, dim3(NT), lds, stream, p, vpad, DS, fuse);                           \
+            TLLM_HGRN_K(DT, 8);                                                                                                     \
         else if (dsz == 16)                                                                                                         \
-            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 16>), hg, dim3(NT), lds, stream, p, vpad, DS, fuse);                          \
+            TLLM_HGRN_K(DT, 16);                                                                                                    \
         else                                                                                                                        \
-            hipLaunchKernelGGL((hgrn2_head_kernel<DT, 32>), hg, dim3(NT), lds, stream, p, vpad, DS, fuse);                          \
+            TLLM_HGRN_K(DT, 32);                                                                                                    \
     } while (0)
             if (p.dtype == DT_BF16)
                 TLLM_HGRN_H(DT_BF16);
             else
                 TLLM_HGRN_H(DT_FLOAT);
 #undef TLLM_HGRN_H
+#undef TLLM_HGRN_K
             if (launched("stack_hgrn2 (sliced)"))
                 return -1;
             if (fuse)

@@ -368,7 +368,7 @@ tllm_stack_t tllm_stack_create(const char* config_text)
         else
         {
             if (!stack_hgrn2_serves(l.dim, l.vdim))
-                return fail("hgrn2: dim up to 2048");
+                return fail("hgrn2: dim up to 512");
             l.n_q = l.heads * l.dim;
             l.n_k = l.heads * l.dim; // forget gate
             l.n_v = l.heads * l.vdim;
