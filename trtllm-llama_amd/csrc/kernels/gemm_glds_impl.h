@@ -185,7 +185,7 @@ __global__ __launch_bounds__(64 * (WM * WN * KG + LW)) void gemm_glds_kernel(con
                 acc[i][j][r] = 0;
 
     const int fr = lane & 31, fk = lane >> 5;
-    const bool vec_out = p.out_dtype == (WT == W_BF16 ? DT_BFLOAT16 : DT_HALF) && !p.resid && !(p.ldc & 7) && !(N & 7) && !(reinterpret_cast<uintptr_t>(p.c) & 15)
+    const bool vec_out = p.out_dtype == (WT == W_BF16 ? DT_BFLOAT16 : DT_HALF) && !p.resid && !p.bias && !p.act && !(p.ldc & 7) && !(N & 7) && !(reinterpret_cast<uintptr_t>(p.c) & 15)
         && !(reinterpret_cast<uintptr_t>(p.residual) & 15);
     if constexpr (LW > 0)
     {
@@ -464,10 +464,20 @@ __global__ __launch_bounds__(64 * (WM * WN * KG + LW)) void gemm_glds_kernel(con
                         }
                         p.resid[(int64_t) row * p.ldr + col] += g * v;
                     }
-                    else if (p.out_dtype == DT_BFLOAT16)
-                        reinterpret_cast<uint16_t*>(p.c)[o] = f2bf(v);
                     else
-                        reinterpret_cast<float*>(p.c)[o] = v;
+                    {
+                        float u = p.bias ? v + p.bias[col] : v;
+                        if (p.act == 1)
+                        {
+                            u = p.out_dtype == DT_BFLOAT16 ? bf2f(f2bf(u)) : u;
+                            u = fmaxf(u, 0.f);
+                            u *= u;
+                        }
+                        if (p.out_dtype == DT_BFLOAT16)
+                            reinterpret_cast<uint16_t*>(p.c)[o] = f2bf(u);
+                        else
+                            reinterpret_cast<float*>(p.c)[o] = u;
+                    }
                 }
                 else
                 {

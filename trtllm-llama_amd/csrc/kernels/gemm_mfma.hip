@@ -280,10 +280,20 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
                         }
                         p.resid[(int64_t) row * p.ldr + col] += g * v;
                     }
-                    else if (p.out_dtype == DT_BFLOAT16)
-                        reinterpret_cast<uint16_t*>(p.c)[o] = f2bf(v);
                     else
-                        reinterpret_cast<float*>(p.c)[o] = v;
+                    {
+                        float u = p.bias ? v + p.bias[col] : v;
+                        if (p.act == 1)
+                        {
+                            u = p.out_dtype == DT_BFLOAT16 ? bf2f(f2bf(u)) : u;
+                            u = fmaxf(u, 0.f);
+                            u *= u;
+                        }
+                        if (p.out_dtype == DT_BFLOAT16)
+                            reinterpret_cast<uint16_t*>(p.c)[o] = f2bf(u);
+                        else
+                            reinterpret_cast<float*>(p.c)[o] = u;
+                    }
                 }
                 else
                 {

@@ -359,6 +359,9 @@ struct GemmParams
     const void* gate = nullptr;
     int64_t ldg = 0;
     const float* gate_bias = nullptr;
+    // W_BF16 only, without resid: + bias[n] (fp32 [N]) on the accumulator; act 1: max(v, 0)^2 of the value rounded to the output type
+    const float* bias = nullptr;
+    int32_t act = 0;
     // microbench hook (tllm_gemm_set_clock_probe), set by the launchers only: 2 x uint64 per workgroup {shader cycles, 100 MHz ticks}
     void* clock_probe = nullptr;
     // split-K-2 forms of gemm_sqp.hip (r06), set by the launcher only: per tile two slabs of AH x BN accumulators + two flag words

@@ -665,6 +665,7 @@ size_t stack_attn_workspace_floats(int32_t heads, int32_t maps, int32_t vdim)
 bool stack_attention_tiled(const StackAttnParams& p)
 {
     return p.dtype == DT_BF16 && (p.dim == 32 || p.dim == 64 || p.dim == 128) && (p.vdim == 32 || p.vdim == 64 || p.vdim == 128)
+        && !p.temp && !p.slope && !p.log_r1 && p.mask == MASK_CAUSAL && p.weights == WEIGHTS_SOFTMAX && !p.sink && !p.out_gate
         && p.page % 32 == 0 && p.max_count > 0 && p.entries > 0 && !(reinterpret_cast<uintptr_t>(p.q) & 15)
         && !(reinterpret_cast<uintptr_t>(p.k_pool) & 15) && !(reinterpret_cast<uintptr_t>(p.v_pool) & 7);
 }

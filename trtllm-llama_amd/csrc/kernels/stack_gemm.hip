@@ -44,17 +44,43 @@ __device__ __forceinline__ void seam(const StackGemmParams& p, int row, int col,
         }
         p.resid[(int64_t) row * p.ldr + col] += g * v;
     }
-    else if (p.out_f32 || DT == DT_FLOAT)
-        reinterpret_cast<float*>(p.c)[(int64_t) row * p.ldc + col] = v;
     else
-        reinterpret_cast<uint16_t*>(p.c)[(int64_t) row * p.ldc + col] = f2bf(v);
+    {
+        const bool narrow = !(p.out_f32 || DT == DT_FLOAT);
+        if (p.bias)
+            v += p.bias[col];
+        if (p.act == ACT_RELU2)
+        {
+            v = narrow ? bf2f(f2bf(v)) : v; // the projection's value in its element type, then its activation
+            v = fmaxf(v, 0.f);
+            v *= v;
+        }
+        if (narrow)
+            reinterpret_cast<uint16_t*>(p.c)[(int64_t) row * p.ldc + col] = f2bf(v);
+        else
+            reinterpret_cast<float*>(p.c)[(int64_t) row * p.ldc + col] = v;
+    }
+}
+
+// operands of product blockIdx.z of a batched launch
+template <int DT>
+__device__ __forceinline__ StackGemmParams batch_slice(StackGemmParams p)
+{
+    const int64_t b = blockIdx.z;
+    constexpr int ES = DT == DT_BF16 ? 2 : 4;
+    p.a = reinterpret_cast<const char*>(p.a) + b * p.stride_a * ES;
+    p.w = reinterpret_cast<const char*>(p.w) + b * p.stride_w * ES;
+    if (p.c)
+        p.c = reinterpret_cast<char*>(p.c) + b * p.stride_c * ((p.out_f32 || DT == DT_FLOAT) ? 4 : 2);
+    return p;
 }
 
 constexpr int TM = 64, TN = 64, TK = 16;
 
 template <int DT>
-__global__ __launch_bounds__(256) void fma_tile_kernel(const StackGemmParams p)
+__global__ __launch_bounds__(256) void fma_tile_kernel(const StackGemmParams p_in)
 {
+    const StackGemmParams p = batch_slice<DT>(p_in);
     __shared__ float As[TK][TM + 4];
     __shared__ float Ws[TK][TN + 4];
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
@@ -108,8 +134,9 @@ __global__ __launch_bounds__(256) void fma_tile_kernel(const StackGemmParams p)
 constexpr int SK_R = 2;
 
 template <int MR>
-__global__ __launch_bounds__(256) void skinny_kernel(const StackGemmParams p)
+__global__ __launch_bounds__(256) void skinny_kernel(const StackGemmParams p_in)
 {
+    const StackGemmParams p = batch_slice<DT_BF16>(p_in);
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     const int n0 = (blockIdx.x * 4 + wid) * SK_R;
     if (n0 >= p.N)
@@ -218,16 +245,22 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
         set_error("stack_gemm: element type %d is not served (bfloat16 or float32)", p.dtype);
         return -1;
     }
-    const dim3 tiles((p.N + TN - 1) / TN, (p.M + TM - 1) / TM);
+    if (p.batch < 1 || (p.batch > 1 && p.resid))
+    {
+        set_error("stack_gemm: batch %d (a batched product has no residual seam)", p.batch);
+        return -1;
+    }
+    const dim3 tiles((p.N + TN - 1) / TN, (p.M + TM - 1) / TM, p.batch);
     if (p.dtype == DT_FLOAT)
     {
         hipLaunchKernelGGL((fma_tile_kernel<DT_FLOAT>), tiles, dim3(256), 0, stream, p);
         return launched("stack_gemm fp32");
     }
-    const bool aligned = !(reinterpret_cast<uintptr_t>(p.a) & 15) && !(reinterpret_cast<uintptr_t>(p.w) & 15) && p.K % 8 == 0 && p.lda % 8 == 0;
+    const bool aligned = !(reinterpret_cast<uintptr_t>(p.a) & 15) && !(reinterpret_cast<uintptr_t>(p.w) & 15) && p.K % 8 == 0 && p.lda % 8 == 0
+        && (p.batch == 1 || (p.stride_a % 8 == 0 && p.stride_w % 8 == 0));
     if (aligned && p.M <= 8)
     {
-        const dim3 grid((p.N + 4 * SK_R - 1) / (4 * SK_R));
+        const dim3 grid((p.N + 4 * SK_R - 1) / (4 * SK_R), 1, p.batch);
         if (p.M <= 1)
             hipLaunchKernelGGL((skinny_kernel<1>), grid, dim3(256), 0, stream, p);
         else if (p.M <= 4)
@@ -238,26 +271,34 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
     }
     if (aligned)
     {
-        GemmParams g;
-        g.wtype = W_BF16;
-        g.out_dtype = p.out_f32 ? DT_FLOAT : DT_BFLOAT16;
-        g.M = p.M;
-        g.N = p.N;
-        g.K = p.K;
-        g.a = p.a;
-        g.lda = p.lda;
-        g.w = p.w;
-        g.ldw = (int64_t) p.K * 2;
-        g.c = p.c;
-        g.ldc = p.ldc;
-        g.resid = p.resid;
-        g.ldr = p.ldr;
-        g.gate = p.gate;
-        g.ldg = p.ldg;
-        g.gate_bias = p.gate_bias;
-        if (p.M >= 32 && p.K % 64 == 0)
-            return launch_glds_bf16(g, stream);
-        const int rc = launch_gemm_mfma(g, stream);
+        // the MFMA tile kernels take one product per launch: a batch is a sequence of launches
+        int rc = 0;
+        for (int b = 0; b < p.batch && rc == 0; ++b)
+        {
+            GemmParams g;
+            g.wtype = W_BF16;
+            g.out_dtype = p.out_f32 ? DT_FLOAT : DT_BFLOAT16;
+            g.M = p.M;
+            g.N = p.N;
+            g.K = p.K;
+            g.a = reinterpret_cast<const char*>(p.a) + (int64_t) b * p.stride_a * 2;
+            g.lda = p.lda;
+            g.w = reinterpret_cast<const char*>(p.w) + (int64_t) b * p.stride_w * 2;
+            g.ldw = (int64_t) p.K * 2;
+            g.c = p.c ? reinterpret_cast<char*>(p.c) + (int64_t) b * p.stride_c * (p.out_f32 ? 4 : 2) : nullptr;
+            g.ldc = p.ldc;
+            g.resid = p.resid;
+            g.ldr = p.ldr;
+            g.gate = p.gate;
+            g.ldg = p.ldg;
+            g.gate_bias = p.gate_bias;
+            g.bias = p.bias;
+            g.act = p.act;
+            if (p.M >= 32 && p.K % 64 == 0)
+                rc = launch_glds_bf16(g, stream);
+            else
+                rc = launch_gemm_mfma(g, stream);
+        }
         if (rc <= 0)
             return rc;
     }

@@ -23,8 +23,13 @@ constexpr int32_t DT_BF16 = 7; // nvinfer1::DataType::kBF16
 //   dtype DT_BF16: MFMA tiles (gemm_mfma.hip, v_mfma_f32_32x32x16_bf16) for M > 8, the streaming skinny kernel below it;
 //   dtype DT_FLOAT: fp32 FMA tiles (stack_gemm.hip).
 // Epilogue, when `resid` is set: resid[m, n] += sigmoid(gate[m, n] + gate_bias[n]) * C[m, n]  (fp32 residual stream, the
-// sublayer's gate taken from another projection's columns); nothing is written to `c` then.
+// sublayer's gate taken from another projection's columns); nothing is written to `c` then.  Otherwise `bias` (fp32 [N]) is added
+// to the accumulator and `act` is applied to the value rounded to the element type: ACT_RELU2 = max(v, 0)^2.
+// `batch` > 1: that many independent products of the same shape, operand b at a + b * stride_a (elements) and so on - the
+// per-head products of latent attention (one weight block per head over one slice of a shared row).
 // ---------------------------------------------------------------------------------------------
+constexpr int32_t ACT_NONE = 0, ACT_RELU2 = 1;
+
 struct StackGemmParams
 {
     int32_t dtype = DT_BF16;     // element type of a, w (and of c unless out_f32)
@@ -40,15 +45,20 @@ struct StackGemmParams
     const void* gate = nullptr;  // element type `dtype`, [M, ldg]: pre-activation of the gate (null: plain accumulate into resid)
     int64_t ldg = 0;
     const float* gate_bias = nullptr; // fp32 [N] or null
+    const float* bias = nullptr;      // fp32 [N] or null (no resid)
+    int32_t act = ACT_NONE;           // (no resid)
+    int32_t batch = 1;
+    int64_t stride_a = 0, stride_w = 0, stride_c = 0; // elements, between the operands of consecutive products
 };
 int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream);
 
 // ---------------------------------------------------------------------------------------------
 // Pointwise pieces.
 // ---------------------------------------------------------------------------------------------
-// x[t, :] = table[ids[t], :] * scale (fp32 residual stream); keep (optional) receives the same rows
+// x[t, :] = table[ids[t], :] * scale (fp32 residual stream); keep (optional) receives the same rows; copies > 1: the row is also
+// written to x + c * copy_stride, c < copies (residual streams that all start from the embedding output)
 int launch_stack_embed(float* x, float* keep, const int32_t* ids, const void* table, int32_t dtype, int32_t tokens, int32_t width,
-    int32_t vocab, float scale, hipStream_t stream);
+    int32_t vocab, float scale, hipStream_t stream, int32_t copies = 1, int64_t copy_stride = 0);
 // x[t, :] += (add ? add[t, :] : 0) + (row ? row[:] : 0): the entry of a pass over a looped layer range
 int launch_stack_pass_entry(float* x, const float* add, const float* row, int32_t tokens, int32_t width, hipStream_t stream);
 // RMS norm in `groups` equal consecutive parts of the row, every part divided by its own sqrt(mean(part^2) + eps); the two
@@ -56,6 +66,29 @@ int launch_stack_pass_entry(float* x, const float* add, const float* row, int32_
 // gather (row r reads x[rows[r]]).  y2 / w2 may be null.
 int launch_stack_group_rmsnorm(void* y1, void* y2, const float* x, const int32_t* rows, const float* w1, const float* w2, int32_t dtype,
     int32_t n_rows, int32_t width, int32_t groups, float eps, hipStream_t stream);
+// Hyper-connected residual streams xs[s] = x + s * stream_stride (fp32 [tokens, width] each, `streams` >= 1 of them; one stream with
+// mix = out = in = 1 is the plain residual sum).  In one pass over a row:
+//   1. y != null: a sublayer's result lands, all streams at once from the old ones: xs[t] <- sum_s mix[s * streams + t] xs[s] + out[t] y
+//   2. u = sum_s in[s] xs[s]  (in == null: the plain sum)
+//   3. h != null: h = u / sqrt(mean(u^2) + eps) * w   (element type `dtype`: the next sublayer's input)
+//      sum_out != null: sum_out = u (fp32)
+// Everything is fp32 but h.  mix / out / in are device arrays.
+struct StackHyperParams
+{
+    int32_t dtype = DT_BF16;
+    int32_t tokens = 0, width = 0, streams = 1;
+    float* x = nullptr;
+    int64_t stream_stride = 0;
+    const float* y = nullptr;   // [tokens, width] or null
+    const float* mix = nullptr; // [streams, streams], indexed [from, to]
+    const float* out = nullptr; // [streams]
+    const float* in = nullptr;  // [streams] or null
+    void* h = nullptr;
+    const float* w = nullptr;   // [width] norm weight as applied (any offset already added)
+    float eps = 1e-5f;
+    float* sum_out = nullptr;
+};
+int launch_stack_hyper_norm(const StackHyperParams& p, hipStream_t stream);
 // y[t, c] = gelu_tanh(gu[t, c]) * gu[t, ff + c] over a [tokens, ld] projection that holds gate then up columns
 int launch_stack_gelu_gate(void* y, const void* gu, int32_t dtype, int32_t tokens, int32_t ff, int64_t ld, hipStream_t stream);
 
@@ -77,6 +110,26 @@ struct StackAttnParams
     // maps == 2: o = a1 - lambda * a2; head_norm: o /= sqrt(mean(o^2) + eps) over vdim, then * out_scale
     float lambda = 0.f, out_scale = 1.f, eps = 1e-5f;
     int32_t head_norm = 0;
+    // Per-head numbers, fp32 [heads] on the device, null = absent.  With i the row's position and j the key's:
+    //   score = q.k * scale (soft cap) * temp[h] - slope[h] * (i - j) - log_r1[h] * ln(1 + log_r2[h] * (i - j))
+    const float* temp = nullptr;
+    const float* slope = nullptr;
+    const float* log_r1 = nullptr;
+    const float* log_r2 = nullptr;
+    // mask: which keys j <= i a row sees.  MASK_WINDOW: i - j < mask_size; MASK_CHUNK: floor(i / mask_size) == floor(j / mask_size)
+    int32_t mask = 0, mask_size = 0;
+    // weights: WEIGHTS_SOFTMAX, its denominator also holding exp(sink[h]) when sink is set (a logit without key or value);
+    // WEIGHTS_SIGMOID: weight = sigmoid(score + wbias[h]) per key, not normalised over keys
+    int32_t weights = 0;
+    const float* sink = nullptr;
+    const float* wbias = nullptr;
+    // the head's output times sigmoid(out_gate[t * ld_gate + h]) (pre-activations in the element type), null = none
+    const void* out_gate = nullptr;
+    int64_t ld_gate = 0;
+    // the projection's rows before anything else: + bias (fp32 [q | k | v columns]), then q and k of every head and map divided by
+    // their root mean square over dim (qk_unit_norm, eps)
+    const float* bias = nullptr;
+    int32_t qk_unit_norm = 0;
     const void* proj = nullptr; // [tokens, ldp]: q rows (heads * maps * dim), k rows (kv_heads * maps * dim), v rows (kv_heads * vdim)
     int64_t ldp = 0;
     void* q = nullptr;          // scratch [tokens, heads * maps * dim]: rotated queries
@@ -94,6 +147,8 @@ struct StackAttnParams
     void* out = nullptr;                  // [tokens, heads * vdim]
     float* split_ws = nullptr;            // decoding steps: partials of the cross-workgroup key split (stack_attn_workspace_floats); null: no split
 };
+constexpr int32_t MASK_CAUSAL = 0, MASK_WINDOW = 1, MASK_CHUNK = 2;
+constexpr int32_t WEIGHTS_SOFTMAX = 0, WEIGHTS_SIGMOID = 1;
 // rotates q and k, appends k and v of the step's rows to the paged cache
 int launch_stack_rope_kv(const StackAttnParams& p, hipStream_t stream);
 // causal attention of the step's rows over their sequences' cache (which already holds the step's own keys)
@@ -101,6 +156,20 @@ int launch_stack_attention(const StackAttnParams& p, hipStream_t stream);
 size_t stack_attn_workspace_floats(int32_t heads, int32_t maps, int32_t vdim); // floats of split_ws a layer of this shape needs
 // frequencies of the rotation with YaRN-style scaling (factor <= 0: none): fills freq[dims / 2], returns the cos / sin multiplier
 float stack_rope_freqs(float* freq, int32_t dims, double base, double factor, double original, double fast, double slow);
+
+// ---------------------------------------------------------------------------------------------
+// Latent attention: a token leaves one latent c [rank] (RMS-normed with a plain weight) and one rotated key part [rot] that all
+// heads share; a head's unrotated key is W_uk c and its value W_uv c.  The cache holds c and the rotated part only, and attention
+// runs in the absorbed form: with a = W_uk^T q_plain (per head, [rank]) the score is a.c + q_rot.k_rot, and the head's output is
+// W_uv (sum_j p_j c_j).  That is launch_stack_attention with one key/value head of dim = rank + rot and vdim = rank:
+//   K pool rows [c | k_rot], V pool rows c, queries [a | q_rot].
+// This kernel does the pointwise part for the step's rows; the two per-head products around the attention are batched
+// launch_stack_gemm calls.  proj [tokens, ldp]: q (heads * (dim + rot): per head plain then rotated part), then rank + rot columns.
+// It writes the rotated q part into q_abs[t, h, rank : rank + rot] and appends the token to the cache; a.dim = rank + rot,
+// a.vdim = rank, a.kv_heads = 1, a.rot_dims = how many of the rot dimensions turn (pairs (2i, 2i + 1), the rest pass), a.freq,
+// a.q = q_abs and the pools are read from `a`.
+// ---------------------------------------------------------------------------------------------
+int launch_stack_latent_prep(const StackAttnParams& a, int32_t qk_dim, const float* latent_norm_w, hipStream_t stream);
 
 // ---------------------------------------------------------------------------------------------
 // HGRN2: per head a state S [dim, vdim] (fp32, one per sequence slot), S <- diag(f) S + (1 - f) v^T, o = S^T q with

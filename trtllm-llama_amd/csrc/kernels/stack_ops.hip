@@ -67,7 +67,7 @@ inline bool known_dtype(int32_t dt, const char* what)
 // ------------------------------------------------------------------------------------------------------------ pointwise
 template <int DT>
 __global__ __launch_bounds__(256) void embed_kernel(float* x, float* keep, const int32_t* ids, const void* table, int width, int vocab,
-    float scale)
+    float scale, int copies, int64_t copy_stride)
 {
     const int t = blockIdx.x;
     int id = ids[t];
@@ -75,10 +75,77 @@ __global__ __launch_bounds__(256) void embed_kernel(float* x, float* keep, const
     for (int c = threadIdx.x; c < width; c += blockDim.x)
     {
         const float v = El<DT>::ld(table, (int64_t) id * width + c) * scale;
-        x[(int64_t) t * width + c] = v;
+        for (int k = 0; k < copies; ++k)
+            x[k * copy_stride + (int64_t) t * width + c] = v;
         if (keep)
             keep[(int64_t) t * width + c] = v;
     }
+}
+
+// Hyper-connected residual streams: one workgroup per row; the combined row u stays in LDS between the sum of squares and the
+// scaling, the streams are read and written once.
+constexpr int HY_T = 256, HY_MAXS = 8;
+
+template <int DT>
+__global__ __launch_bounds__(HY_T) void hyper_norm_kernel(const StackHyperParams p)
+{
+    extern __shared__ float u_s[]; // [width]
+    __shared__ float red[32];
+    __shared__ float cm[HY_MAXS * HY_MAXS], co[HY_MAXS], ci[HY_MAXS];
+    const int t = blockIdx.x, tid = threadIdx.x, S = p.streams;
+    if (tid < S * S)
+        cm[tid] = p.y ? p.mix[tid] : 0.f;
+    if (tid < S)
+    {
+        co[tid] = p.y ? p.out[tid] : 0.f;
+        ci[tid] = p.in ? p.in[tid] : 1.f;
+    }
+    __syncthreads();
+    float ss = 0.f;
+    for (int c = tid; c < p.width; c += HY_T)
+    {
+        const int64_t o = (int64_t) t * p.width + c;
+        float xs[HY_MAXS], u = 0.f;
+#pragma unroll
+        for (int s = 0; s < HY_MAXS; ++s)
+            xs[s] = s < S ? p.x[s * p.stream_stride + o] : 0.f;
+        if (p.y)
+        {
+            const float y = p.y[o];
+#pragma unroll
+            for (int to = 0; to < HY_MAXS; ++to)
+            {
+                if (to < S)
+                {
+                    float a = 0.f;
+#pragma unroll
+                    for (int s = 0; s < HY_MAXS; ++s)
+                        if (s < S)
+                            a = fmaf(cm[s * S + to], xs[s], a);
+                    a = fmaf(co[to], y, a);
+                    p.x[to * p.stream_stride + o] = a;
+                    u = fmaf(ci[to], a, u);
+                }
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int s = 0; s < HY_MAXS; ++s)
+                if (s < S)
+                    u = fmaf(ci[s], xs[s], u);
+        }
+        if (p.sum_out)
+            p.sum_out[o] = u;
+        u_s[c] = u;
+        ss += u * u;
+    }
+    if (!p.h)
+        return;
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float) p.width + p.eps);
+    for (int c = tid; c < p.width; c += HY_T)
+        El<DT>::st(p.h, (int64_t) t * p.width + c, u_s[c] * inv * p.w[c]);
 }
 
 __global__ __launch_bounds__(256) void pass_entry_kernel(float* x, const float* add, const float* row, int64_t n, int width)
@@ -197,6 +264,138 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(const StackAttnParams p)
     }
 }
 
+// The general form of the step before attention: one wave per (row, vector), a vector being one map of one query head, one map of
+// one key head, or one value head.  Projection bias, unit RMS of q and k over dim (fp32), rotation of neighbouring pairs (the
+// partner sits in the neighbouring lane), then the store into the query scratch or the page.  dim, vdim <= 64 * PREP_EPL.
+constexpr int PREP_EPL = 8;
+
+template <int DT>
+__global__ __launch_bounds__(256) void attn_prep_kernel(const StackAttnParams p)
+{
+    const int t = blockIdx.x, lane = threadIdx.x & 63;
+    const int vec = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int D = p.dim, nqv = p.heads * p.maps, nkv = p.kv_heads * p.maps;
+    if (vec >= nqv + nkv + p.kv_heads)
+        return;
+    const int e = p.tok_entry[t], pos = p.tok_pos[t];
+    const int blk = p.block_table[(int64_t) e * p.max_blocks + pos / p.page], off = pos % p.page;
+    const int64_t row = (int64_t) t * p.ldp;
+    if (vec >= nqv + nkv)
+    {
+        const int g = vec - nqv - nkv, col0 = (nqv + nkv) * D + g * p.vdim;
+        for (int c = lane; c < p.vdim; c += 64)
+        {
+            float v = El<DT>::ld(p.proj, row + col0 + c);
+            if (p.bias)
+                v += p.bias[col0 + c];
+            El<DT>::st(p.v_pool, (((int64_t) blk * p.kv_heads + g) * p.vdim + c) * p.page + off, v);
+        }
+        return;
+    }
+    const int col0 = vec * D;
+    float v[PREP_EPL], ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < PREP_EPL; ++k)
+    {
+        const int d = lane + 64 * k;
+        v[k] = 0.f;
+        if (d < D)
+        {
+            v[k] = El<DT>::ld(p.proj, row + col0 + d);
+            if (p.bias)
+                v[k] += p.bias[col0 + d];
+            if (DT == DT_BF16 && p.bias)
+                v[k] = bf2f(f2bf(v[k])); // the biased projection is a value of the element type
+        }
+        ss += v[k] * v[k];
+    }
+    float inv = 1.f;
+    if (p.qk_unit_norm)
+        inv = 1.f / sqrtf(wave_sum(ss) / (float) D + p.eps);
+#pragma unroll
+    for (int k = 0; k < PREP_EPL; ++k)
+    {
+        const int d = lane + 64 * k;
+        float x = v[k] * inv;
+        const float other = __shfl_xor(x, 1, 64); // pairs (2i, 2i + 1): lane parity = dimension parity
+        if (d < p.rot_dims)
+        {
+            float sn, cs;
+            sincosf((float) pos * p.freq[d >> 1], &sn, &cs);
+            sn *= p.mscale;
+            cs *= p.mscale;
+            x = (d & 1) ? x * cs + other * sn : x * cs - other * sn;
+        }
+        if (d < D)
+        {
+            if (vec < nqv)
+                El<DT>::st(p.q, (int64_t) t * nqv * D + col0 + d, x);
+            else
+                El<DT>::st(p.k_pool, (((int64_t) blk * nkv + (vec - nqv)) * p.page + off) * D + d, x);
+        }
+    }
+}
+
+// Latent attention, the pointwise part: per row the latent's RMS norm (plain weight) and the rotation of the shared key part into
+// the page ([c | k_rot] as the key row, c channel-major as the value row), and the rotation of every head's rotated query part into
+// the absorbed query [a | q_rot] (the `a` part is a product of its own).  One wave per (row, head) plus one per row for the latent.
+template <int DT>
+__global__ __launch_bounds__(256) void latent_prep_kernel(const StackAttnParams p, int qk_dim, const float* norm_w)
+{
+    const int t = blockIdx.x, lane = threadIdx.x & 63;
+    const int vec = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (vec > p.heads)
+        return;
+    const int C = p.vdim, R = p.dim - C, pos = p.tok_pos[t]; // of the R dimensions of the rotated part the first rot_dims turn
+    const int64_t row = (int64_t) t * p.ldp;
+    if (vec < p.heads)
+    {
+        const int64_t src = row + (int64_t) vec * (qk_dim + R) + qk_dim;
+        for (int d = lane; d < R; d += 64)
+        {
+            float x = El<DT>::ld(p.proj, src + d);
+            if (d < p.rot_dims)
+            {
+                const float other = El<DT>::ld(p.proj, src + (d ^ 1));
+                float sn, cs;
+                sincosf((float) pos * p.freq[d >> 1], &sn, &cs);
+                x = (d & 1) ? x * cs + other * sn : x * cs - other * sn;
+            }
+            El<DT>::st(p.q, ((int64_t) t * p.heads + vec) * p.dim + C + d, x);
+        }
+        return;
+    }
+    const int e = p.tok_entry[t];
+    const int blk = p.block_table[(int64_t) e * p.max_blocks + pos / p.page], off = pos % p.page;
+    const int64_t src = row + (int64_t) p.heads * (qk_dim + R);
+    float ss = 0.f;
+    for (int c = lane; c < C; c += 64)
+    {
+        const float x = El<DT>::ld(p.proj, src + c);
+        ss += x * x;
+    }
+    const float inv = 1.f / sqrtf(wave_sum(ss) / (float) C + p.eps);
+    const int64_t krow = ((int64_t) blk * p.page + off) * p.dim;
+    for (int c = lane; c < C; c += 64)
+    {
+        const float x = El<DT>::ld(p.proj, src + c) * inv * norm_w[c];
+        El<DT>::st(p.k_pool, krow + c, x);
+        El<DT>::st(p.v_pool, ((int64_t) blk * C + c) * p.page + off, x);
+    }
+    for (int d = lane; d < R; d += 64)
+    {
+        float x = El<DT>::ld(p.proj, src + C + d);
+        if (d < p.rot_dims)
+        {
+            const float other = El<DT>::ld(p.proj, src + C + (d ^ 1));
+            float sn, cs;
+            sincosf((float) pos * p.freq[d >> 1], &sn, &cs);
+            x = (d & 1) ? x * cs + other * sn : x * cs - other * sn;
+        }
+        El<DT>::st(p.k_pool, krow + C + d, x);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ attention, general form
 // One workgroup per (row, head): scores of 128 keys at a time by one thread per key, online softmax per map, P V by one thread
 // per value channel.  Any dim / vdim <= 512, both element types; the tiled kernels of stack_attn.hip take the shapes they serve.
@@ -228,7 +427,17 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
     }
     __syncthreads();
     const int nkeys = pos + 1;
-    for (int k0 = 0; k0 < nkeys; k0 += AT)
+    // the first key the mask lets this row see: a window's lower edge, the start of the row's chunk
+    int k_lo = 0;
+    if (p.mask == MASK_WINDOW)
+        k_lo = pos - p.mask_size + 1 > 0 ? pos - p.mask_size + 1 : 0;
+    else if (p.mask == MASK_CHUNK)
+        k_lo = pos / p.mask_size * p.mask_size;
+    const float temp = p.temp ? p.temp[h] : 1.f, slope = p.slope ? p.slope[h] : 0.f;
+    const float r1 = p.log_r1 ? p.log_r1[h] : 0.f, r2 = p.log_r1 ? p.log_r2[h] : 0.f;
+    const bool sigm = p.weights == WEIGHTS_SIGMOID;
+    const float wb = sigm && p.wbias ? p.wbias[h] : 0.f;
+    for (int k0 = k_lo; k0 < nkeys; k0 += AT)
     {
         const int kj = k0 + tid;
         float s[MAPS];
@@ -247,6 +456,11 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
                 a *= p.scale;
                 if (p.softcap > 0.f)
                     a = p.softcap * tanhf(a / p.softcap);
+                a *= temp;
+                const float dist = (float) (pos - kj);
+                a -= slope * dist;
+                if (p.log_r1)
+                    a -= r1 * logf(1.f + r2 * dist);
                 s[m] = a;
             }
         }
@@ -261,6 +475,13 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
 #pragma unroll
         for (int m = 0; m < MAPS; ++m)
         {
+            if (sigm)
+            {
+                // every key's weight stands alone: no running maximum, no denominator
+                corr[m] = 1.f;
+                ps[m * AT + tid] = kj < nkeys ? 1.f / (1.f + expf(-(s[m] + wb))) : 0.f;
+                continue;
+            }
             const float bm = block_max(s[m], red);
             const float mn = fmaxf(m_run[m], bm);
             corr[m] = expf(m_run[m] - mn); // 0 at the first block
@@ -295,6 +516,25 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
         }
         __syncthreads();
     }
+    float fin[MAPS]; // what turns a map's accumulator into its output
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+    {
+        if (sigm)
+            fin[m] = 1.f;
+        else if (p.sink)
+        {
+            // the sink joins the denominator like one more key with this logit, and brings no value
+            const float sk = p.sink[h], mf = fmaxf(m_run[m], sk);
+            const float w_keys = expf(m_run[m] - mf);
+            fin[m] = w_keys / (l_run[m] * w_keys + expf(sk - mf));
+        }
+        else
+            fin[m] = 1.f / l_run[m];
+    }
+    float og = 1.f;
+    if (p.out_gate)
+        og = 1.f / (1.f + expf(-El<DT>::ld(p.out_gate, (int64_t) t * p.ld_gate + h)));
     float o[A_CPT], ss = 0.f;
 #pragma unroll
     for (int c = 0; c < A_CPT; ++c)
@@ -302,9 +542,9 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
         o[c] = 0.f;
         if (tid + c * AT < V)
         {
-            o[c] = acc[0][c] / l_run[0];
+            o[c] = acc[0][c] * fin[0];
             if (MAPS == 2)
-                o[c] -= p.lambda * (acc[MAPS - 1][c] / l_run[MAPS - 1]);
+                o[c] -= p.lambda * (acc[MAPS - 1][c] * fin[MAPS - 1]);
             ss += o[c] * o[c];
         }
     }
@@ -317,7 +557,7 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
 #pragma unroll
     for (int c = 0; c < A_CPT; ++c)
         if (tid + c * AT < V)
-            El<DT>::st(p.out, ((int64_t) t * p.heads + h) * V + tid + c * AT, o[c] * mul);
+            El<DT>::st(p.out, ((int64_t) t * p.heads + h) * V + tid + c * AT, o[c] * mul * og);
 }
 
 // ------------------------------------------------------------------------------------------------------------------ HGRN2
@@ -572,17 +812,43 @@ __global__ __launch_bounds__(256) void head_rmsnorm_kernel(void* y, const float*
 
 // ---------------------------------------------------------------------------------------------------------------- launchers
 int launch_stack_embed(float* x, float* keep, const int32_t* ids, const void* table, int32_t dtype, int32_t tokens, int32_t width,
-    int32_t vocab, float scale, hipStream_t stream)
+    int32_t vocab, float scale, hipStream_t stream, int32_t copies, int64_t copy_stride)
 {
     if (tokens <= 0)
         return 0;
     if (!known_dtype(dtype, "stack_embed"))
         return -1;
     if (dtype == DT_BF16)
-        hipLaunchKernelGGL((embed_kernel<DT_BF16>), dim3(tokens), dim3(256), 0, stream, x, keep, ids, table, width, vocab, scale);
+        hipLaunchKernelGGL((embed_kernel<DT_BF16>), dim3(tokens), dim3(256), 0, stream, x, keep, ids, table, width, vocab, scale, copies,
+            copy_stride);
     else
-        hipLaunchKernelGGL((embed_kernel<DT_FLOAT>), dim3(tokens), dim3(256), 0, stream, x, keep, ids, table, width, vocab, scale);
+        hipLaunchKernelGGL((embed_kernel<DT_FLOAT>), dim3(tokens), dim3(256), 0, stream, x, keep, ids, table, width, vocab, scale, copies,
+            copy_stride);
     return launched("stack_embed");
+}
+
+int launch_stack_hyper_norm(const StackHyperParams& p, hipStream_t stream)
+{
+    if (p.tokens <= 0)
+        return 0;
+    if (!known_dtype(p.dtype, "stack_hyper_norm"))
+        return -1;
+    if (p.streams < 1 || p.streams > HY_MAXS || p.width < 1 || !p.x || (p.y && (!p.mix || !p.out)) || (p.h && !p.w))
+    {
+        set_error("stack_hyper_norm: %d streams (1 .. %d) of width %d, or a missing operand", p.streams, HY_MAXS, p.width);
+        return -1;
+    }
+    const size_t lds = sizeof(float) * (size_t) p.width;
+    if (lds > 64 * 1024)
+    {
+        set_error("stack_hyper_norm: width %d is beyond the row it keeps in LDS", p.width);
+        return -1;
+    }
+    if (p.dtype == DT_BF16)
+        hipLaunchKernelGGL((hyper_norm_kernel<DT_BF16>), dim3(p.tokens), dim3(HY_T), lds, stream, p);
+    else
+        hipLaunchKernelGGL((hyper_norm_kernel<DT_FLOAT>), dim3(p.tokens), dim3(HY_T), lds, stream, p);
+    return launched("stack_hyper_norm");
 }
 
 int launch_stack_pass_entry(float* x, const float* add, const float* row, int32_t tokens, int32_t width, hipStream_t stream)
@@ -644,6 +910,12 @@ static bool attn_shape_ok(const StackAttnParams& p, const char* what)
         set_error("%s: the rotation pairs neighbours: dim %d and rot_dims %d must be even, rot_dims <= dim", what, p.dim, p.rot_dims);
         return false;
     }
+    if (p.mask < MASK_CAUSAL || p.mask > MASK_CHUNK || (p.mask != MASK_CAUSAL && p.mask_size < 1) || p.weights < WEIGHTS_SOFTMAX
+        || p.weights > WEIGHTS_SIGMOID || (p.log_r1 && !p.log_r2))
+    {
+        set_error("%s: mask %d of size %d, weights %d is not a form it serves", what, p.mask, p.mask_size, p.weights);
+        return false;
+    }
     return true;
 }
 
@@ -653,6 +925,21 @@ int launch_stack_rope_kv(const StackAttnParams& p, hipStream_t stream)
         return 0;
     if (!attn_shape_ok(p, "stack_rope_kv"))
         return -1;
+    if (p.bias || p.qk_unit_norm)
+    {
+        if (p.dim > 64 * PREP_EPL)
+        {
+            set_error("stack_rope_kv: dim %d is beyond the %d a wave keeps", p.dim, 64 * PREP_EPL);
+            return -1;
+        }
+        const int vecs = (p.heads + p.kv_heads) * p.maps + p.kv_heads;
+        const dim3 pg(p.tokens, (vecs + 3) / 4);
+        if (p.dtype == DT_BF16)
+            hipLaunchKernelGGL((attn_prep_kernel<DT_BF16>), pg, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((attn_prep_kernel<DT_FLOAT>), pg, dim3(256), 0, stream, p);
+        return launched("stack_rope_kv (general)");
+    }
     // few rows (decoding): one element per thread; many rows: a workgroup per row walks it
     const int per_row = (p.heads + p.kv_heads) * p.maps * p.dim;
     const dim3 grid(p.tokens, p.tokens >= 64 ? 1 : (per_row + 255) / 256);
@@ -661,6 +948,26 @@ int launch_stack_rope_kv(const StackAttnParams& p, hipStream_t stream)
     else
         hipLaunchKernelGGL((rope_kv_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, p);
     return launched("stack_rope_kv");
+}
+
+int launch_stack_latent_prep(const StackAttnParams& p, int32_t qk_dim, const float* latent_norm_w, hipStream_t stream)
+{
+    if (p.tokens <= 0)
+        return 0;
+    if (!attn_shape_ok(p, "stack_latent_prep"))
+        return -1;
+    if (p.kv_heads != 1 || p.maps != 1 || p.rot_dims > p.dim - p.vdim || p.vdim < 1 || qk_dim < 1 || !latent_norm_w || !p.freq)
+    {
+        set_error("stack_latent_prep: one key/value head of dim = rank + rotated part and vdim = rank (dim %d, vdim %d, rot %d, kv_heads %d, maps %d)",
+            p.dim, p.vdim, p.rot_dims, p.kv_heads, p.maps);
+        return -1;
+    }
+    const dim3 grid(p.tokens, (p.heads + 1 + 3) / 4);
+    if (p.dtype == DT_BF16)
+        hipLaunchKernelGGL((latent_prep_kernel<DT_BF16>), grid, dim3(256), 0, stream, p, qk_dim, latent_norm_w);
+    else
+        hipLaunchKernelGGL((latent_prep_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, p, qk_dim, latent_norm_w);
+    return launched("stack_latent_prep");
 }
 
 int launch_stack_attention_general(const StackAttnParams& p, hipStream_t stream)

@@ -7,7 +7,13 @@
 //   x += sigmoid(P1[rg1] + b1) * (ctx Wo^T)                      product with the gated-residual seam in its epilogue
 //   P2 = h2 [Wgate; Wup; Wrg2]^T ; a = gelu(P2[gate]) * P2[up]
 //   x += sigmoid(P2[rg2] + b2) * (a Wdown^T)
-// on the packed rows of the step.  The residual stream x is fp32 in both element types.
+// on the packed rows of the step (block=parallel, residual=gated).  With block=sequential, residual=hyper a layer run is pre-norm
+// with `streams` hyper-connected copies of the residual:
+//   h1 = norm1(sum_s in1[s] x_s)                                  one launch, which also lands the sublayer before it (below)
+//   P1 = h1 [Wq; Wk; Wv; Wg]^T  (latent attention: [Wq; Wdkv])    mixer as above, per-head output gate inside the attention launch
+//   y = ctx Wo^T (fp32);  x_t <- sum_s mix1[s, t] x_s + out1[t] y   folded into the next launch that reads the streams
+//   h2 = norm2(sum_s in2[s] x_s);  a = relu(h2 Wup^T)^2 (product epilogue);  y = a Wdown^T;  x_t <- sum_s mix2[s, t] x_s + out2[t] y
+// The residual streams are fp32 in both element types.
 #include "../../../include/tllm_stack_api.h"
 #include "../kernels/stack_kernels.h"
 #include <cmath>
@@ -39,7 +45,17 @@ struct HostTensor
 enum MixerKind
 {
     MIX_ATTENTION = 0,
-    MIX_HGRN2 = 1
+    MIX_HGRN2 = 1,
+    MIX_LATENT = 2
+};
+enum MlpKind
+{
+    MLP_GELU_GATE = 0, // W_down (gelu_tanh(W_gate h) * W_up h)
+    MLP_RELU2 = 1      // W_down relu(W_up h)^2
+};
+struct HyperW
+{
+    float *mix = nullptr, *out = nullptr, *in = nullptr;
 };
 
 struct Layer
@@ -52,10 +68,19 @@ struct Layer
     // derived
     int n_q = 0, n_k = 0, n_v = 0, n_mix = 0, n_ctx = 0; // columns of P1: q | k (or f) | v | rg1
     float lambda = 0.f, mscale = 1.f;
+    int mlp = MLP_GELU_GATE;
+    int qkv_bias = 0, qk_norm = 0, head_temp = 0, pos_bias = 0 /* 0 none, 1 linear, 2 log */, mask = MASK_CAUSAL, mask_size = 0,
+        weights = WEIGHTS_SOFTMAX, sink = 0, out_gate = 0;
+    double slope_base = 8;
+    int kv_rank = 0, rot_part = 0;  // latent attention: rank of the latent, size of the shared rotated key part (rot_dims of it turn)
+    int n_gate = 0, n_rg = 0;       // further columns of P1: per-head output gates, the gated residual's projection
+    int n_lat = 0;                  // latent attention: heads * kv_rank
     // device
-    void *w_mix = nullptr, *w_o = nullptr, *w_gu = nullptr, *w_down = nullptr;
+    void *w_mix = nullptr, *w_o = nullptr, *w_gu = nullptr, *w_down = nullptr, *w_ukT = nullptr, *w_uv = nullptr;
     float *norm1 = nullptr, *norm2 = nullptr, *rg1_b = nullptr, *rg2_b = nullptr, *f_bias = nullptr, *lower = nullptr, *hnorm = nullptr,
-          *freq = nullptr;
+          *freq = nullptr, *bias = nullptr, *temp = nullptr, *slope = nullptr, *r1 = nullptr, *r2 = nullptr, *sinkv = nullptr, *wbias = nullptr,
+          *lat_norm = nullptr;
+    HyperW hc[2];
 };
 
 struct Run
@@ -75,6 +100,9 @@ struct tllm_stack
     int dtype = DT_BF16, es = 2;
     int width = 0, vocab = 0, groups = 1, page = 64, blocks = 0, slots = 0, taps = 0;
     int loop_start = 0, loop_stop = 0, loop_times = 1;
+    bool sequential = false, hyper = false;
+    int streams = 1;
+    float norm_offset = 0.f, *ones = nullptr;
     float eps = 1e-5f, emb_scale = 1.f;
     std::vector<Layer> layers;
     std::vector<Run> runs;
@@ -85,10 +113,10 @@ struct tllm_stack
     std::vector<void*> owned;
     // scratch, grown to the largest step seen
     int cap_tokens = 0, cap_want = 0, cap_ints = 0;
-    float *x = nullptr, *x0 = nullptr, *o32 = nullptr, *logits = nullptr, *tap = nullptr;
-    void *h1 = nullptr, *h2 = nullptr, *proj = nullptr, *q = nullptr, *ctx = nullptr, *act = nullptr, *hw = nullptr;
+    float *x = nullptr, *x0 = nullptr, *o32 = nullptr, *logits = nullptr, *tap = nullptr, *y32 = nullptr;
+    void *h1 = nullptr, *h2 = nullptr, *proj = nullptr, *q = nullptr, *ctx = nullptr, *act = nullptr, *hw = nullptr, *lat = nullptr;
     int32_t *ints = nullptr, *ids_out = nullptr, *pinned = nullptr;
-    int max_proj = 0, max_q = 0, max_ctx = 0, max_ff = 0;
+    int max_proj = 0, max_q = 0, max_ctx = 0, max_ff = 0, max_lat = 0;
     int tap_tokens = 0;
 
     ~tllm_stack()
@@ -101,12 +129,12 @@ struct tllm_stack
     }
     void free_scratch()
     {
-        void* all[] = {x, x0, o32, logits, tap, h1, h2, proj, q, ctx, act, hw, ints, ids_out};
+        void* all[] = {x, x0, o32, logits, tap, y32, h1, h2, proj, q, ctx, act, hw, lat, ints, ids_out};
         for (void* p : all)
             if (p)
                 (void) hipFree(p);
-        x = x0 = o32 = logits = tap = nullptr;
-        h1 = h2 = proj = q = ctx = act = hw = nullptr;
+        x = x0 = o32 = logits = tap = y32 = nullptr;
+        h1 = h2 = proj = q = ctx = act = hw = lat = nullptr;
         ints = ids_out = nullptr;
     }
 };
@@ -236,7 +264,9 @@ int ensure_scratch(tllm_stack* s, int tokens, int want, int n_ints)
         const size_t T = (size_t) std::max(tokens, s->cap_tokens), W = (size_t) std::max(want, s->cap_want);
         const size_t NI = (size_t) std::max(n_ints, s->cap_ints);
         const size_t es = s->es, wd = s->width;
-        HIP_OK(hipMalloc((void**) &s->x, T * wd * 4));
+        HIP_OK(hipMalloc((void**) &s->x, T * wd * 4 * (size_t) s->streams));
+        HIP_OK(hipMalloc((void**) &s->y32, T * wd * 4));
+        HIP_OK(hipMalloc(&s->lat, T * std::max(s->max_lat, 1) * es));
         HIP_OK(hipMalloc((void**) &s->x0, T * wd * 4));
         HIP_OK(hipMalloc((void**) &s->o32, T * std::max(s->max_ctx, 1) * 4));
         HIP_OK(hipMalloc((void**) &s->logits, W * s->vocab * 4));
@@ -308,6 +338,11 @@ tllm_stack_t tllm_stack_create(const char* config_text)
     s->loop_start = geti(s, "loop_start", 0);
     s->loop_stop = geti(s, "loop_stop", 0);
     s->loop_times = geti(s, "loop_times", 1);
+    s->norm_offset = (float) getd(s, "norm_offset", 0.0);
+    s->streams = geti(s, "streams", 1);
+    const std::string block = gets(s, "block", "parallel"), residual = gets(s, "residual", "gated");
+    s->sequential = block == "sequential";
+    s->hyper = residual == "hyper";
     const int L = geti(s, "num_layers", 0);
     auto fail = [&](const char* why) {
         set_error("tllm_stack_create: %s", why);
@@ -320,6 +355,12 @@ tllm_stack_t tllm_stack_create(const char* config_text)
         return fail("width must split into norm_groups equal parts");
     if (s->page < 1 || s->blocks < 1 || s->slots < 1)
         return fail("page_size, num_blocks and num_slots must be positive");
+    if ((block != "parallel" && block != "sequential") || (residual != "gated" && residual != "hyper") || s->sequential != s->hyper)
+        return fail("block=parallel goes with residual=gated, block=sequential with residual=hyper");
+    if (s->streams < 1 || s->streams > 8 || (!s->hyper && s->streams != 1))
+        return fail("streams: 1 to 8, more than one only with residual=hyper");
+    if (s->hyper && s->loop_stop > s->loop_start)
+        return fail("looped layers are built for the gated residual only");
     if (s->loop_times < 1 || s->loop_start < 0 || s->loop_stop < s->loop_start || s->loop_stop > L)
         return fail("the loop must satisfy 0 <= loop_start <= loop_stop <= num_layers, loop_times >= 1");
     s->layers.resize(L);
@@ -332,9 +373,11 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.kind = MIX_ATTENTION;
         else if (kind == "hgrn2")
             l.kind = MIX_HGRN2;
+        else if (kind == "latent_attention")
+            l.kind = MIX_LATENT;
         else
         {
-            set_error("tllm_stack_create: layer %d has mixer type '%s' (attention | hgrn2)", i, kind.c_str());
+            set_error("tllm_stack_create: layer %d has mixer type '%s' (attention | latent_attention | hgrn2)", i, kind.c_str());
             delete s;
             return nullptr;
         }
@@ -345,8 +388,51 @@ tllm_stack_t tllm_stack_create(const char* config_text)
         if (l.heads < 1 || l.dim < 1 || l.vdim < 1 || l.ff < 0)
             return fail("a layer needs heads, dim and vdim");
         l.n_ctx = l.heads * l.vdim;
-        if (l.kind == MIX_ATTENTION)
+        const std::string mlp = gets(s, p + "mlp", "gelu_gate");
+        if (mlp != "gelu_gate" && mlp != "relu2")
+            return fail("a layer's mlp is gelu_gate or relu2");
+        l.mlp = mlp == "relu2" ? MLP_RELU2 : MLP_GELU_GATE;
+        if (l.mlp == MLP_RELU2 && !s->sequential)
+            return fail("the relu2 feed-forward is built for block=sequential");
+        l.n_rg = s->hyper ? 0 : s->width;
+        if (l.kind == MIX_LATENT)
         {
+            l.kv_rank = geti(s, p + "kv_rank", 0);
+            l.rot_part = geti(s, p + "rot_dim", 0);
+            l.rot_dims = geti(s, p + "rot_dims", l.rot_part);
+            l.rot_base = getd(s, p + "rot_base", 10000);
+            l.scale = getd(s, p + "scale", 1.0 / std::sqrt((double) (l.dim + l.rot_part)));
+            if (l.kv_rank < 1 || l.rot_part < 0 || l.rot_dims < 0 || (l.rot_dims & 1) || l.rot_dims > l.rot_part || ((l.kv_rank + l.rot_part) & 1))
+                return fail("latent_attention: kv_rank positive, rot_dims even and <= rot_dim, kv_rank + rot_dim even");
+            l.kv_heads = 1;
+            l.n_q = l.heads * (l.dim + l.rot_part);
+            l.n_k = l.kv_rank + l.rot_part; // the down projection: latent | rotated key part
+            l.n_v = 0;
+            l.n_lat = l.heads * l.kv_rank;
+            s->max_lat = std::max(s->max_lat, l.n_lat);
+            s->max_q = std::max(s->max_q, l.heads * (l.kv_rank + l.rot_part));
+        }
+        else if (l.kind == MIX_ATTENTION)
+        {
+            l.qkv_bias = geti(s, p + "qkv_bias", 0);
+            l.qk_norm = geti(s, p + "qk_norm", 0);
+            l.head_temp = geti(s, p + "head_temp", 0);
+            const std::string pb = gets(s, p + "pos_bias", "none"), mk = gets(s, p + "mask", "causal"), wt = gets(s, p + "weights", "softmax");
+            if ((pb != "none" && pb != "linear" && pb != "log") || (mk != "causal" && mk != "window" && mk != "chunk")
+                || (wt != "softmax" && wt != "sigmoid"))
+                return fail("attention: pos_bias none | linear | log, mask causal | window | chunk, weights softmax | sigmoid");
+            l.pos_bias = pb == "linear" ? 1 : (pb == "log" ? 2 : 0);
+            l.slope_base = getd(s, p + "slope_base", 8.0);
+            l.mask = mk == "window" ? MASK_WINDOW : (mk == "chunk" ? MASK_CHUNK : MASK_CAUSAL);
+            l.mask_size = geti(s, p + "mask_size", 0);
+            l.weights = wt == "sigmoid" ? WEIGHTS_SIGMOID : WEIGHTS_SOFTMAX;
+            l.sink = geti(s, p + "sink", 0);
+            l.out_gate = geti(s, p + "out_gate", 0);
+            if (l.mask != MASK_CAUSAL && l.mask_size < 1)
+                return fail("attention: a window or chunk mask needs mask_size >= 1");
+            if (l.sink && l.weights == WEIGHTS_SIGMOID)
+                return fail("attention: a sink belongs to softmax weights");
+            l.n_gate = l.out_gate ? l.heads : 0;
             l.kv_heads = geti(s, p + "kv_heads", l.heads);
             l.maps = geti(s, p + "maps", 1);
             l.diff = getd(s, p + "diff", 0);
@@ -373,8 +459,8 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.n_k = l.heads * l.dim; // forget gate
             l.n_v = l.heads * l.vdim;
         }
-        l.n_mix = l.n_q + l.n_k + l.n_v + s->width;
-        s->max_proj = std::max(s->max_proj, std::max(l.n_mix, 2 * l.ff + s->width));
+        l.n_mix = l.n_q + l.n_k + l.n_v + l.n_rg + l.n_gate;
+        s->max_proj = std::max(s->max_proj, std::max(l.n_mix, (l.mlp == MLP_RELU2 ? l.ff : 2 * l.ff) + l.n_rg));
         s->max_q = std::max(s->max_q, l.n_q);
         s->max_ctx = std::max(s->max_ctx, l.n_ctx);
         s->max_ff = std::max(s->max_ff, l.ff);
@@ -447,9 +533,27 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
     t = need(s, "head", {s->vocab, Wd});
     if (!t || upload_rows(s, {t}, &s->head))
         return -1;
-    t = need(s, "final.norm", {Wd});
-    if (!t || upload_f32(s, t->v.data(), t->v.size(), &s->final_norm))
+    // a norm weight as the kernels apply it: the stored value plus the design's offset (0, or 1 for weights stored around zero)
+    auto norm_vec = [&](const std::string& name, int64_t len, float** out) {
+        const HostTensor* v = need(s, name, {len});
+        if (!v)
+            return -1;
+        std::vector<float> w(v->v);
+        for (float& f : w)
+            f += s->norm_offset;
+        return upload_f32(s, w.data(), w.size(), out);
+    };
+    auto norm_plain = [&](const std::string& name, int64_t len, float** out) {
+        const HostTensor* v = need(s, name, {len});
+        return (!v || upload_f32(s, v->v.data(), v->v.size(), out)) ? -1 : 0;
+    };
+    if (norm_vec("final.norm", Wd, &s->final_norm))
         return -1;
+    {
+        const std::vector<float> one(64, 1.f);
+        if (upload_f32(s, one.data(), one.size(), &s->ones))
+            return -1;
+    }
     if (s->loop_stop > s->loop_start)
     {
         t = need(s, "loop.step", {s->loop_times, Wd});
@@ -464,23 +568,80 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
             const HostTensor* v = need(s, p + n, {len});
             return (!v || upload_f32(s, v->v.data(), v->v.size(), out)) ? -1 : 0;
         };
-        if (vec("norm1", Wd, &l.norm1) || vec("rg1.b", Wd, &l.rg1_b))
+        if (norm_vec(p + "norm1", Wd, &l.norm1))
             return -1;
-        const HostTensor* rg1 = need(s, p + "rg1", {Wd, Wd});
+        const HostTensor* rg1 = nullptr;
+        if (!s->hyper)
+        {
+            rg1 = need(s, p + "rg1", {Wd, Wd});
+            if (!rg1 || vec("rg1.b", Wd, &l.rg1_b))
+                return -1;
+        }
+        else
+        {
+            // hyper-connections of the two sublayers; a model with one plain stream has no such tensors: mix = out = in = 1
+            for (int q = 0; q < 2; ++q)
+            {
+                HyperW& hw = l.hc[q];
+                const std::string hp = "hc" + std::to_string(q + 1) + ".";
+                if (s->host.count(p + hp + "mix") == 0 && s->streams == 1)
+                {
+                    hw.mix = hw.out = hw.in = s->ones;
+                    continue;
+                }
+                if (q == 1 && l.ff == 0)
+                    continue;
+                const HostTensor* m = need(s, p + hp + "mix", {s->streams, s->streams});
+                if (!m || upload_f32(s, m->v.data(), m->v.size(), &hw.mix) || vec(hp + "out", s->streams, &hw.out)
+                    || vec(hp + "in", s->streams, &hw.in))
+                    return -1;
+            }
+        }
         const HostTensor* wq = need(s, p + "mix.q", {l.n_q, Wd});
-        const HostTensor* wk = need(s, p + (l.kind == MIX_ATTENTION ? "mix.k" : "mix.f"), {l.n_k, Wd});
-        const HostTensor* wv = need(s, p + "mix.v", {l.n_v, Wd});
+        const HostTensor* wk = need(s, p + (l.kind == MIX_ATTENTION ? "mix.k" : (l.kind == MIX_LATENT ? "mix.dkv" : "mix.f")), {l.n_k, Wd});
+        const HostTensor* wv = l.kind == MIX_LATENT ? nullptr : need(s, p + "mix.v", {l.n_v, Wd});
         const HostTensor* wo = need(s, p + "mix.o", {Wd, l.n_ctx});
-        if (!rg1 || !wq || !wk || !wv || !wo)
+        const HostTensor* wg = l.n_gate ? need(s, p + "mix.g", {l.n_gate, Wd}) : nullptr;
+        if (!wq || !wk || (!wv && l.kind != MIX_LATENT) || !wo || (l.n_gate && !wg))
             return -1;
-        if (upload_rows(s, {wq, wk, wv, rg1}, &l.w_mix) || upload_rows(s, {wo}, &l.w_o))
-            return -1;
-        if (l.kind == MIX_ATTENTION)
+        {
+            std::vector<const HostTensor*> rows = {wq, wk};
+            if (wv)
+                rows.push_back(wv);
+            if (rg1)
+                rows.push_back(rg1);
+            if (wg)
+                rows.push_back(wg);
+            if (upload_rows(s, rows, &l.w_mix) || upload_rows(s, {wo}, &l.w_o))
+                return -1;
+        }
+        if (l.kind == MIX_ATTENTION || l.kind == MIX_LATENT)
         {
             std::vector<float> fr((size_t) std::max(l.rot_dims / 2, 1));
             l.mscale = stack_rope_freqs(fr.data(), l.rot_dims, l.rot_base, l.rot_factor, l.rot_original, l.rot_fast, l.rot_slow);
             if (upload_f32(s, fr.data(), fr.size(), &l.freq))
                 return -1;
+        }
+        if (l.kind == MIX_LATENT)
+        {
+            const int64_t C = l.kv_rank, D = l.dim, E = l.vdim, H = l.heads;
+            const HostTensor* uk = need(s, p + "mix.uk", {H * D, C});
+            const HostTensor* uv = need(s, p + "mix.uv", {H * E, C});
+            if (!uk || !uv || norm_plain(p + "mix.dkv.norm", C, &l.lat_norm))
+                return -1;
+            // W_uk^T per head, [kv_rank, dim]: the query side of the absorbed score is a product with these rows
+            HostTensor tr;
+            tr.dims = {H * C, D};
+            tr.v.resize((size_t) (H * C * D));
+            for (int64_t h = 0; h < H; ++h)
+                for (int64_t d = 0; d < D; ++d)
+                    for (int64_t c = 0; c < C; ++c)
+                        tr.v[(size_t) ((h * C + c) * D + d)] = uk->v[(size_t) ((h * D + d) * C + c)];
+            if (upload_rows(s, {&tr}, &l.w_ukT) || upload_rows(s, {uv}, &l.w_uv))
+                return -1;
+        }
+        else if (l.kind == MIX_ATTENTION)
+        {
             l.lambda = 0.f;
             if (l.maps == 2)
             {
@@ -496,6 +657,33 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
                 }
                 l.lambda = std::exp(d1) - std::exp(d2) + (float) l.diff;
             }
+            if (l.qkv_bias)
+            {
+                const HostTensor *bq = need(s, p + "mix.q.b", {l.n_q}), *bk = need(s, p + "mix.k.b", {l.n_k}), *bv = need(s, p + "mix.v.b", {l.n_v});
+                if (!bq || !bk || !bv)
+                    return -1;
+                std::vector<float> b(bq->v);
+                b.insert(b.end(), bk->v.begin(), bk->v.end());
+                b.insert(b.end(), bv->v.begin(), bv->v.end());
+                if (upload_f32(s, b.data(), b.size(), &l.bias))
+                    return -1;
+            }
+            if (l.head_temp && vec("mix.temp", l.heads, &l.temp))
+                return -1;
+            if (l.pos_bias == 1)
+            {
+                std::vector<float> sl((size_t) l.heads);
+                for (int h = 0; h < l.heads; ++h)
+                    sl[(size_t) h] = (float) std::exp2(-l.slope_base * (h + 1) / l.heads);
+                if (upload_f32(s, sl.data(), sl.size(), &l.slope))
+                    return -1;
+            }
+            if (l.pos_bias == 2 && (vec("mix.r1", l.heads, &l.r1) || vec("mix.r2", l.heads, &l.r2)))
+                return -1;
+            if (l.sink && vec("mix.sink", l.heads, &l.sinkv))
+                return -1;
+            if (l.weights == WEIGHTS_SIGMOID && vec("mix.pb", l.heads, &l.wbias))
+                return -1;
         }
         else
         {
@@ -504,15 +692,27 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
         }
         if (l.ff > 0)
         {
-            if (vec("norm2", Wd, &l.norm2) || vec("rg2.b", Wd, &l.rg2_b))
+            if (norm_vec(p + "norm2", Wd, &l.norm2))
                 return -1;
-            const HostTensor* rg2 = need(s, p + "rg2", {Wd, Wd});
-            const HostTensor* wg = need(s, p + "mlp.gate", {l.ff, Wd});
+            const HostTensor* rg2 = nullptr;
+            if (!s->hyper)
+            {
+                rg2 = need(s, p + "rg2", {Wd, Wd});
+                if (!rg2 || vec("rg2.b", Wd, &l.rg2_b))
+                    return -1;
+            }
+            const HostTensor* wgt = l.mlp == MLP_GELU_GATE ? need(s, p + "mlp.gate", {l.ff, Wd}) : nullptr;
             const HostTensor* wu = need(s, p + "mlp.up", {l.ff, Wd});
             const HostTensor* wd = need(s, p + "mlp.down", {Wd, l.ff});
-            if (!rg2 || !wg || !wu || !wd)
+            if ((l.mlp == MLP_GELU_GATE && !wgt) || !wu || !wd)
                 return -1;
-            if (upload_rows(s, {wg, wu, rg2}, &l.w_gu) || upload_rows(s, {wd}, &l.w_down))
+            std::vector<const HostTensor*> rows;
+            if (wgt)
+                rows.push_back(wgt);
+            rows.push_back(wu);
+            if (rg2)
+                rows.push_back(rg2);
+            if (upload_rows(s, rows, &l.w_gu) || upload_rows(s, {wd}, &l.w_down))
                 return -1;
         }
     }
@@ -520,6 +720,8 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
     for (const Layer& l : s->layers)
         if (l.kind == MIX_ATTENTION)
             ws_floats = std::max(ws_floats, stack_attn_workspace_floats(l.heads, l.maps, l.vdim));
+        else if (l.kind == MIX_LATENT)
+            ws_floats = std::max(ws_floats, stack_attn_workspace_floats(l.heads, 1, l.kv_rank));
     if (ws_floats)
     {
         void* ws = nullptr;
@@ -530,7 +732,14 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
     for (Run& r : s->runs)
     {
         const Layer& l = s->layers[r.layer];
-        if (l.kind == MIX_ATTENTION)
+        if (l.kind == MIX_LATENT)
+        {
+            // one key row [latent | rotated part] and one value row (the latent, channel-major) per token, shared by all heads
+            if (alloc_zero(s, (size_t) s->blocks * s->page * (l.kv_rank + l.rot_part) * s->es, &r.k_pool)
+                || alloc_zero(s, (size_t) s->blocks * s->page * l.kv_rank * s->es, &r.v_pool))
+                return -1;
+        }
+        else if (l.kind == MIX_ATTENTION)
         {
             if (alloc_zero(s, (size_t) s->blocks * l.kv_heads * l.maps * s->page * l.dim * s->es, &r.k_pool)
                 || alloc_zero(s, (size_t) s->blocks * l.kv_heads * s->page * l.vdim * s->es, &r.v_pool))
@@ -650,19 +859,14 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
 
     const int Wd = s->width;
     const bool looped = s->loop_stop > s->loop_start;
-    if (launch_stack_embed(s->x, looped && s->loop_times > 1 ? s->x0 : nullptr, d_tok, s->embed, s->dtype, T, Wd, s->vocab, s->emb_scale, stream))
+    const int64_t stream_stride = (int64_t) T * Wd;
+    if (launch_stack_embed(s->x, looped && s->loop_times > 1 ? s->x0 : nullptr, d_tok, s->embed, s->dtype, T, Wd, s->vocab, s->emb_scale, stream,
+            s->streams, stream_stride))
         return -1;
     s->tap_tokens = T;
-    for (size_t ri = 0; ri < s->runs.size(); ++ri)
-    {
-        const Run& r = s->runs[ri];
-        const Layer& l = s->layers[r.layer];
-        if (r.enters_pass
-            && launch_stack_pass_entry(s->x, r.pass > 0 ? s->x0 : nullptr, s->loop_step + (size_t) r.pass * Wd, T, Wd, stream))
-            return -1;
-        if (launch_stack_group_rmsnorm(s->h1, l.ff > 0 ? s->h2 : nullptr, s->x, nullptr, l.norm1, l.norm2, s->dtype, T, Wd, s->groups, s->eps,
-                stream))
-            return -1;
+
+    // P1 = h1 W_mix^T, then the mixer: its context rows land in s->ctx
+    auto run_mixer = [&](const Layer& l, const Run& r) -> int {
         StackGemmParams g;
         g.dtype = s->dtype;
         g.M = T;
@@ -675,47 +879,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         g.ldc = l.n_mix;
         if (launch_stack_gemm(g, stream))
             return -1;
-        if (l.kind == MIX_ATTENTION)
-        {
-            StackAttnParams a;
-            a.dtype = s->dtype;
-            a.tokens = T;
-            a.entries = E;
-            a.heads = l.heads;
-            a.kv_heads = l.kv_heads;
-            a.maps = l.maps;
-            a.dim = l.dim;
-            a.vdim = l.vdim;
-            a.rot_dims = l.rot_dims;
-            a.freq = l.freq;
-            a.mscale = l.mscale;
-            a.scale = (float) l.scale;
-            a.softcap = (float) l.softcap;
-            a.lambda = l.lambda;
-            a.out_scale = (float) (1.0 - l.diff);
-            a.eps = s->eps;
-            a.head_norm = l.head_norm;
-            a.proj = s->proj;
-            a.ldp = l.n_mix;
-            a.q = s->q;
-            a.k_pool = r.k_pool;
-            a.v_pool = r.v_pool;
-            a.page = s->page;
-            a.max_blocks = MB;
-            a.block_table = d_table;
-            a.tok_entry = d_tent;
-            a.tok_pos = d_tpos;
-            a.ent_first = d_first;
-            a.ent_count = d_count;
-            a.ent_pos0 = d_pos0;
-            a.max_count = max_count;
-            a.max_context = max_ctx;
-            a.out = s->ctx;
-            a.split_ws = s->attn_ws;
-            if (launch_stack_rope_kv(a, stream) || launch_stack_attention(a, stream))
-                return -1;
-        }
-        else
+        if (l.kind == MIX_HGRN2)
         {
             StackHgrnParams hp;
             hp.dtype = s->dtype;
@@ -738,9 +902,210 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
             hp.max_count = max_count;
             hp.o32 = s->o32;
             hp.out = s->ctx;
-            if (launch_stack_hgrn2(hp, stream))
-                return -1;
+            return launch_stack_hgrn2(hp, stream);
         }
+        StackAttnParams a;
+        a.dtype = s->dtype;
+        a.tokens = T;
+        a.entries = E;
+        a.heads = l.heads;
+        a.freq = l.freq;
+        a.scale = (float) l.scale;
+        a.eps = s->eps;
+        a.proj = s->proj;
+        a.ldp = l.n_mix;
+        a.q = s->q;
+        a.k_pool = r.k_pool;
+        a.v_pool = r.v_pool;
+        a.page = s->page;
+        a.max_blocks = MB;
+        a.block_table = d_table;
+        a.tok_entry = d_tent;
+        a.tok_pos = d_tpos;
+        a.ent_first = d_first;
+        a.ent_count = d_count;
+        a.ent_pos0 = d_pos0;
+        a.max_count = max_count;
+        a.max_context = max_ctx;
+        a.split_ws = s->attn_ws;
+        if (l.kind == MIX_LATENT)
+        {
+            // absorbed form: one shared key/value head over [latent | rotated part]; queries [W_uk^T q_plain | rotated q part]
+            const int C = l.kv_rank, R = l.rot_part, D = l.dim, H = l.heads;
+            a.kv_heads = 1;
+            a.maps = 1;
+            a.dim = C + R;
+            a.vdim = C;
+            a.rot_dims = l.rot_dims;
+            a.out = s->lat;
+            if (launch_stack_latent_prep(a, D, l.lat_norm, stream))
+                return -1;
+            StackGemmParams qa;
+            qa.dtype = s->dtype;
+            qa.M = T;
+            qa.N = C;
+            qa.K = D;
+            qa.a = s->proj;
+            qa.lda = l.n_mix;
+            qa.w = l.w_ukT;
+            qa.c = s->q;
+            qa.ldc = (int64_t) H * (C + R);
+            qa.batch = H;
+            qa.stride_a = D + R;
+            qa.stride_w = (int64_t) C * D;
+            qa.stride_c = C + R;
+            if (launch_stack_gemm(qa, stream) || launch_stack_attention(a, stream))
+                return -1;
+            StackGemmParams ve; // head h: ctx[:, h] = lat[:, h] W_uv,h^T
+            ve.dtype = s->dtype;
+            ve.M = T;
+            ve.N = l.vdim;
+            ve.K = C;
+            ve.a = s->lat;
+            ve.lda = (int64_t) H * C;
+            ve.w = l.w_uv;
+            ve.c = s->ctx;
+            ve.ldc = l.n_ctx;
+            ve.batch = H;
+            ve.stride_a = C;
+            ve.stride_w = (int64_t) l.vdim * C;
+            ve.stride_c = l.vdim;
+            return launch_stack_gemm(ve, stream);
+        }
+        a.kv_heads = l.kv_heads;
+        a.maps = l.maps;
+        a.dim = l.dim;
+        a.vdim = l.vdim;
+        a.rot_dims = l.rot_dims;
+        a.mscale = l.mscale;
+        a.softcap = (float) l.softcap;
+        a.lambda = l.lambda;
+        a.out_scale = (float) (1.0 - l.diff);
+        a.head_norm = l.head_norm;
+        a.temp = l.temp;
+        a.slope = l.slope;
+        a.log_r1 = l.r1;
+        a.log_r2 = l.r2;
+        a.mask = l.mask;
+        a.mask_size = l.mask_size;
+        a.weights = l.weights;
+        a.sink = l.sinkv;
+        a.wbias = l.wbias;
+        a.bias = l.bias;
+        a.qk_unit_norm = l.qk_norm;
+        if (l.n_gate)
+        {
+            a.out_gate = (const char*) s->proj + (size_t) (l.n_q + l.n_k + l.n_v + l.n_rg) * s->es;
+            a.ld_gate = l.n_mix;
+        }
+        a.out = s->ctx;
+        return (launch_stack_rope_kv(a, stream) || launch_stack_attention(a, stream)) ? -1 : 0;
+    };
+
+    // residual=hyper: the sublayer result in y32 that has not yet been folded into the streams, and the launch that folds it,
+    // combines the streams for the next reader and norms the combination
+    const HyperW* pending = nullptr;
+    auto hyper = [&](const float* in, void* h, const float* w, float* sum_out) -> int {
+        StackHyperParams hp;
+        hp.dtype = s->dtype;
+        hp.tokens = T;
+        hp.width = Wd;
+        hp.streams = s->streams;
+        hp.x = s->x;
+        hp.stream_stride = stream_stride;
+        if (pending)
+        {
+            hp.y = s->y32;
+            hp.mix = pending->mix;
+            hp.out = pending->out;
+        }
+        hp.in = in;
+        hp.h = h;
+        hp.w = w;
+        hp.eps = s->eps;
+        hp.sum_out = sum_out;
+        pending = nullptr;
+        return launch_stack_hyper_norm(hp, stream);
+    };
+
+    for (size_t ri = 0; ri < s->runs.size(); ++ri)
+    {
+        const Run& r = s->runs[ri];
+        const Layer& l = s->layers[r.layer];
+        if (s->hyper)
+        {
+            if (hyper(l.hc[0].in, s->h1, l.norm1, nullptr) || run_mixer(l, r))
+                return -1;
+            StackGemmParams o; // y = ctx Wo^T in fp32: the residual sum is 32-bit
+            o.dtype = s->dtype;
+            o.out_f32 = 1;
+            o.M = T;
+            o.N = Wd;
+            o.K = l.n_ctx;
+            o.a = s->ctx;
+            o.lda = l.n_ctx;
+            o.w = l.w_o;
+            o.c = s->y32;
+            o.ldc = Wd;
+            if (launch_stack_gemm(o, stream))
+                return -1;
+            pending = &l.hc[0];
+            if (l.ff > 0)
+            {
+                if (hyper(l.hc[1].in, s->h1, l.norm2, nullptr))
+                    return -1;
+                StackGemmParams u;
+                u.dtype = s->dtype;
+                u.M = T;
+                u.K = Wd;
+                u.a = s->h1;
+                u.lda = Wd;
+                u.w = l.w_gu;
+                const void* act = s->act;
+                if (l.mlp == MLP_RELU2)
+                {
+                    u.N = l.ff;
+                    u.c = s->act;
+                    u.ldc = l.ff;
+                    u.act = ACT_RELU2;
+                    if (launch_stack_gemm(u, stream))
+                        return -1;
+                }
+                else
+                {
+                    u.N = 2 * l.ff;
+                    u.c = s->proj;
+                    u.ldc = u.N;
+                    if (launch_stack_gemm(u, stream) || launch_stack_gelu_gate(s->act, s->proj, s->dtype, T, l.ff, u.N, stream))
+                        return -1;
+                }
+                StackGemmParams dn;
+                dn.dtype = s->dtype;
+                dn.out_f32 = 1;
+                dn.M = T;
+                dn.N = Wd;
+                dn.K = l.ff;
+                dn.a = act;
+                dn.lda = l.ff;
+                dn.w = l.w_down;
+                dn.c = s->y32;
+                dn.ldc = Wd;
+                if (launch_stack_gemm(dn, stream))
+                    return -1;
+                pending = &l.hc[1];
+            }
+            if (s->taps && hyper(nullptr, nullptr, nullptr, s->tap + ri * (size_t) T * Wd))
+                return -1;
+            continue;
+        }
+        if (r.enters_pass
+            && launch_stack_pass_entry(s->x, r.pass > 0 ? s->x0 : nullptr, s->loop_step + (size_t) r.pass * Wd, T, Wd, stream))
+            return -1;
+        if (launch_stack_group_rmsnorm(s->h1, l.ff > 0 ? s->h2 : nullptr, s->x, nullptr, l.norm1, l.norm2, s->dtype, T, Wd, s->groups, s->eps,
+                stream))
+            return -1;
+        if (run_mixer(l, r))
+            return -1;
         // x += sigmoid(P1[rg1] + b1) * (ctx Wo^T)
         StackGemmParams o;
         o.dtype = s->dtype;
@@ -755,22 +1120,26 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         o.gate = (const char*) s->proj + (size_t) (l.n_q + l.n_k + l.n_v) * s->es;
         o.ldg = l.n_mix;
         o.gate_bias = l.rg1_b;
+        if (launch_stack_gemm(o, stream))
+            return -1;
         if (l.ff > 0)
         {
-            // the feed-forward reads the same x as the mixer: its projection runs before the mixer's update lands (h2 is ready)
+            // the feed-forward reads the same x as the mixer (h2 was normed before the mixer's update landed); P1's columns are
+            // consumed once the mixer and the O product have run, so P2 may take their place
             StackGemmParams u;
             u.dtype = s->dtype;
             u.M = T;
-            u.N = 2 * l.ff + Wd;
             u.K = Wd;
             u.a = s->h2;
             u.lda = Wd;
             u.w = l.w_gu;
-            u.c = s->proj; // P1's columns are consumed once the mixer and the O product have run: keep the order below
+            u.c = s->proj;
+            const int n_act = l.mlp == MLP_RELU2 ? l.ff : 2 * l.ff; // columns ahead of the residual gate's
+            u.N = n_act + Wd;
             u.ldc = u.N;
-            if (launch_stack_gemm(o, stream))
+            if (launch_stack_gemm(u, stream))
                 return -1;
-            if (launch_stack_gemm(u, stream) || launch_stack_gelu_gate(s->act, s->proj, s->dtype, T, l.ff, u.N, stream))
+            if (launch_stack_gelu_gate(s->act, s->proj, s->dtype, T, l.ff, u.N, stream))
                 return -1;
             StackGemmParams dn;
             dn.dtype = s->dtype;
@@ -782,20 +1151,26 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
             dn.w = l.w_down;
             dn.resid = s->x;
             dn.ldr = Wd;
-            dn.gate = (const char*) s->proj + (size_t) (2 * l.ff) * s->es;
+            dn.gate = (const char*) s->proj + (size_t) n_act * s->es;
             dn.ldg = u.N;
             dn.gate_bias = l.rg2_b;
             if (launch_stack_gemm(dn, stream))
                 return -1;
         }
-        else if (launch_stack_gemm(o, stream))
-            return -1;
         if (s->taps)
             HIP_OK(hipMemcpyAsync(s->tap + ri * (size_t) T * Wd, s->x, (size_t) T * Wd * 4, hipMemcpyDeviceToDevice, stream));
     }
+    // the row the final norm reads: the sum of the streams (one stream of the gated residual: x itself)
+    const float* x_final = s->x;
+    if (s->hyper)
+    {
+        if (hyper(nullptr, nullptr, nullptr, s->x0))
+            return -1;
+        x_final = s->x0;
+    }
     if (NW > 0)
     {
-        if (launch_stack_group_rmsnorm(s->hw, nullptr, s->x, d_want, s->final_norm, nullptr, s->dtype, NW, Wd, s->groups, s->eps, stream))
+        if (launch_stack_group_rmsnorm(s->hw, nullptr, x_final, d_want, s->final_norm, nullptr, s->dtype, NW, Wd, s->groups, s->eps, stream))
             return -1;
         StackGemmParams hd;
         hd.dtype = s->dtype;
@@ -856,9 +1231,20 @@ int64_t tllm_stack_step_bytes(tllm_stack_t s, int32_t n_tokens, int64_t context_
     for (const Run& r : s->runs)
     {
         const Layer& l = s->layers[r.layer];
-        bytes += ((int64_t) l.n_mix + l.n_ctx + (l.ff > 0 ? 3 * (int64_t) l.ff + s->width : 0)) * s->width * s->es;
-        if (l.kind == MIX_ATTENTION)
-            bytes += context_tokens * ((int64_t) l.n_k + l.n_v) * s->es;
+        const int64_t ff_rows = l.ff > 0 ? (l.mlp == MLP_RELU2 ? 2 : 3) * (int64_t) l.ff + l.n_rg : 0;
+        bytes += ((int64_t) l.n_mix + l.n_ctx + ff_rows) * s->width * s->es;
+        if (l.kind == MIX_LATENT)
+        {
+            // the two per-head expansions, and per context token the key row [latent | rotated part] and the latent again as value
+            bytes += (int64_t) l.heads * l.kv_rank * (l.dim + l.vdim) * s->es;
+            bytes += context_tokens * (2 * (int64_t) l.kv_rank + l.rot_part) * s->es;
+        }
+        else if (l.kind == MIX_ATTENTION)
+        {
+            // a window or a chunk bounds what a row reads of its context
+            const int64_t ctx = l.mask == MASK_CAUSAL ? context_tokens : std::min<int64_t>(context_tokens, (int64_t) n_entries * l.mask_size);
+            bytes += ctx * ((int64_t) l.n_k + l.n_v) * s->es;
+        }
         else
             bytes += 2 * (int64_t) n_entries * l.heads * l.dim * l.vdim * 4;
     }

@@ -7,11 +7,13 @@ import os
 
 from .llama.model import LLaMAForCausalLM
 from .tolenex.model import TolenexForCausalLM
+from .vetipel.model import VetipelForCausalLM
 
 MODEL_REGISTRY = {
     'LlamaForCausalLM': LLaMAForCausalLM,
     'LLaMAForCausalLM': LLaMAForCausalLM,
     'Tolenex': TolenexForCausalLM,
+    'Vetipel': VetipelForCausalLM,
 }
 
 
