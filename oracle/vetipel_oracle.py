@@ -171,3 +171,17 @@ def forward(cfg, w, tokens):
         taps.append(xs.sum(axis=0))
     x = xs.sum(axis=0)
     return offset_rms_norm(x, w['final.norm'], eps) @ w['head'].T, taps
+
+
+def logits(tokens, w, cfg):
+    return forward(cfg, w, tokens)[0]
+
+
+def greedy(prompt, w, cfg, n_new):
+    """n_new tokens by arg-max, every one from a whole-sequence pass."""
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        nxt = int(np.argmax(logits(toks, w, cfg)[-1]))
+        out.append(nxt)
+        toks.append(nxt)
+    return out

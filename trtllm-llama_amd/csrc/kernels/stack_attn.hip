@@ -56,12 +56,48 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
 
+// What a head does to its raw scores, in the base-2 domain (an exponential is one v_exp_f32, a logarithm one v_log_f32):
+//   score2 = cap(q.k * scale) * temp * log2 e - slope2 * (i - j) - r1 * log2(1 + r2 * (i - j))
+// and how scores become weights: softmax (running maximum and sum), or a sigmoid per key (no state across keys).
+struct HeadMods
+{
+    float scale2, cap2, cap_arg, temp, slope2, r1, r2, wb2;
+    int pen, sigm; // pen: any of temp / slope / r1 is set
+};
+
+__device__ __forceinline__ HeadMods head_mods(const StackAttnParams& p, int h)
+{
+    constexpr float LOG2E = 1.4426950408889634f;
+    HeadMods m;
+    m.temp = p.temp ? p.temp[h] : 1.f;
+    m.scale2 = p.scale * LOG2E * (p.softcap > 0.f ? 1.f : m.temp);
+    m.cap2 = p.softcap > 0.f ? p.softcap * LOG2E * m.temp : 0.f;
+    m.cap_arg = p.softcap > 0.f ? p.scale / p.softcap * 2.f * LOG2E : 0.f;
+    m.slope2 = p.slope ? p.slope[h] * LOG2E : 0.f;
+    m.r1 = p.log_r1 ? p.log_r1[h] : 0.f;
+    m.r2 = p.log_r1 ? p.log_r2[h] : 0.f;
+    m.pen = (p.slope || p.log_r1) ? 1 : 0;
+    m.sigm = p.weights == WEIGHTS_SIGMOID;
+    m.wb2 = m.sigm && p.wbias ? p.wbias[h] * LOG2E : 0.f;
+    return m;
+}
+
+// the first key position a row at `pos` sees
+__device__ __forceinline__ int first_visible(const StackAttnParams& p, int pos)
+{
+    if (p.mask == MASK_WINDOW)
+        return pos - p.mask_size + 1 > 0 ? pos - p.mask_size + 1 : 0;
+    if (p.mask == MASK_CHUNK)
+        return pos / p.mask_size * p.mask_size;
+    return 0;
+}
+
 // Scores of one 32-key block of one map -> its P^T fragment, with the online-softmax state of the lane's query row brought up to
-// date.  Everything in the base-2 domain (scale2 / cap2 carry log2 e), so an exponential is one v_exp_f32.  `masked` is wave-uniform:
-// only blocks that reach past the first row's position compare keys with positions.
+// date.  `masked` is wave-uniform: only blocks that reach past the first row's position, or start before the last row's first
+// visible key, compare keys with positions.
 template <int VT>
-__device__ __forceinline__ uint4 softmax_block(f32x4 (&s)[2], float& m_run, float& l_run, f32x4 (&acc)[VT], float scale2, float cap2,
-    float cap_arg, bool masked, int key_lane0, int qpos)
+__device__ __forceinline__ uint4 softmax_block(f32x4 (&s)[2], float& m_run, float& l_run, f32x4 (&acc)[VT], const HeadMods& hm, bool masked,
+    int key_lane0, int qpos, int klo)
 {
     float bm = -INFINITY;
 #pragma unroll
@@ -70,19 +106,38 @@ __device__ __forceinline__ uint4 softmax_block(f32x4 (&s)[2], float& m_run, floa
         for (int i = 0; i < 4; ++i)
         {
             float v;
-            if (cap2 > 0.f)
+            if (hm.cap2 > 0.f)
             {
                 // cap * tanh(x / cap) with tanh(y) = (e^{2y} - 1) / (e^{2y} + 1); cap_arg = scale / cap * 2 log2 e
-                const float t2 = __builtin_amdgcn_exp2f(fminf(fmaxf(s[t][i] * cap_arg, -43.f), 43.f));
-                v = cap2 * (t2 - 1.f) * __builtin_amdgcn_rcpf(t2 + 1.f);
+                const float t2 = __builtin_amdgcn_exp2f(fminf(fmaxf(s[t][i] * hm.cap_arg, -43.f), 43.f));
+                v = hm.cap2 * (t2 - 1.f) * __builtin_amdgcn_rcpf(t2 + 1.f);
             }
             else
-                v = s[t][i] * scale2;
-            if (masked && key_lane0 + t * 16 + i > qpos)
+                v = s[t][i] * hm.scale2;
+            const int kidx = key_lane0 + t * 16 + i;
+            if (hm.pen)
+            {
+                const float dist = (float) (qpos - kidx);
+                v -= hm.slope2 * dist;
+                if (hm.r1 != 0.f)
+                    v -= hm.r1 * __builtin_amdgcn_logf(fmaxf(1.f + hm.r2 * dist, 1e-30f));
+            }
+            if (masked && (kidx > qpos || kidx < klo))
                 v = -INFINITY;
             s[t][i] = v;
             bm = fmaxf(bm, v);
         }
+    if (hm.sigm)
+    {
+        // every key's weight stands alone: 1 / (1 + 2^-(score2 + offset2)); a hidden key's is 2^-inf = 0
+        float pv[8];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                pv[t * 4 + i] = s[t][i] == -INFINITY ? 0.f : __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-(s[t][i] + hm.wb2)));
+        return make_uint4(pack_bf16(pv[0], pv[1]), pack_bf16(pv[2], pv[3]), pack_bf16(pv[4], pv[5]), pack_bf16(pv[6], pv[7]));
+    }
     bm = rows_max(bm);
     const float mn = fmaxf(m_run, bm);
     const bool none = mn == -INFINITY; // this row sees no key of this block (nor of any before)
@@ -110,6 +165,27 @@ __device__ __forceinline__ uint4 softmax_block(f32x4 (&s)[2], float& m_run, floa
     return make_uint4(pack_bf16(pv[0], pv[1]), pack_bf16(pv[2], pv[3]), pack_bf16(pv[4], pv[5]), pack_bf16(pv[6], pv[7]));
 }
 
+// How a finished row leaves: the softmax denominator also takes the head's sink (a logit without key or value), given the row's
+// running maximum M (base 2) and sum L relative to it -> the factor on the accumulator; sigmoid weights are not normalised.
+__device__ __forceinline__ float finish_factor(const StackAttnParams& p, int h, float M, float L)
+{
+    if (p.weights == WEIGHTS_SIGMOID)
+        return 1.f;
+    if (!p.sink)
+        return 1.f / L;
+    const float sk = p.sink[h] * 1.4426950408889634f, mf = fmaxf(M, sk);
+    const float wk = __builtin_amdgcn_exp2f(M - mf);
+    return wk / (L * wk + __builtin_amdgcn_exp2f(sk - mf));
+}
+
+__device__ __forceinline__ float out_gate_of(const StackAttnParams& p, int64_t t, int h)
+{
+    if (!p.out_gate)
+        return 1.f;
+    const float z = bf2f(reinterpret_cast<const uint16_t*>(p.out_gate)[t * p.ld_gate + h]);
+    return 1.f / (1.f + __expf(-z));
+}
+
 template <int MAPS, int DK, int VT, int NW>
 __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParams p, int below_count, int ks)
 {
@@ -131,14 +207,13 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     const int g = h / (p.heads / p.kv_heads);
     const int page = p.page;
     const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
-    constexpr float LOG2E = 1.4426950408889634f;
-    const float scale2 = p.scale * LOG2E, cap2 = p.softcap > 0.f ? p.softcap * LOG2E : 0.f;
-    const float cap_arg = p.softcap > 0.f ? p.scale / p.softcap * 2.f * LOG2E : 0.f;
+    const HeadMods hm = head_mods(p, h);
     const uint16_t* kp = reinterpret_cast<const uint16_t*>(p.k_pool);
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.v_pool);
 
     const int qrow = r0 + col < count ? r0 + col : count - 1;
     const int qpos = pos0 + qrow;
+    const int klo = first_visible(p, qpos);
     bf16x8 qf[MAPS][DK];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m)
@@ -148,6 +223,8 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
                 reinterpret_cast<const uint16_t*>(p.q) + (((int64_t) (first + qrow) * p.heads + h) * MAPS + m) * D + ks * 32 + 8 * g4));
     const int last_row = r0 + 15 < count ? r0 + 15 : count - 1;
     const int nblk = (pos0 + last_row) / 32 + 1;
+    // the tile's key blocks: from the one that holds the first row's first visible key; klo_last: the last row's (the largest)
+    const int blk_lo = first_visible(p, pos0 + r0) / 32, klo_last = first_visible(p, pos0 + last_row);
 
     float m_run[MAPS], l_run[MAPS];
     f32x4 acc[MAPS][VT];
@@ -177,7 +254,7 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
                     kf[m][t][ks] = *reinterpret_cast<const uint4*>(krow + ks * 32);
             }
     };
-    const int kb0 = split * NW + w, kstep = ks * NW;
+    const int kb0 = blk_lo + split * NW + w, kstep = ks * NW;
     int blk = kb0 < nblk ? table[kb0 * 32 / page] : 0;
     if (kb0 < nblk)
         request_k(kb0, blk);
@@ -211,10 +288,10 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
             request_k(kb + kstep, blk);
         }
         uint4 pf[MAPS]; // P^T fragment of the block, 8 bfloat16 per map
-        const bool masked = key0 + 31 > pos0 + r0; // wave-uniform
+        const bool masked = key0 + 31 > pos0 + r0 || key0 < klo_last; // wave-uniform
 #pragma unroll
         for (int m = 0; m < MAPS; ++m)
-            pf[m] = softmax_block<VT>(s[m], m_run[m], l_run[m], acc[m], scale2, cap2, cap_arg, masked, key0 + 4 * g4, qpos);
+            pf[m] = softmax_block<VT>(s[m], m_run[m], l_run[m], acc[m], hm, masked, key0 + 4 * g4, qpos, klo);
         // O^T += V^T P^T: slot j of the lane's k group is key 4 g4 + j (j < 4) or 16 + 4 g4 + (j - 4) of the block, in both operands
 #pragma unroll
         for (int ct = 0; ct < VT; ++ct)
@@ -259,6 +336,8 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
         {
             const float mw = ml_part[((ww * MAPS + m) * 16 + row) * 2];
             wgt[m][ww] = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M); // the running maxima are base-2 exponents
+            if (hm.sigm)
+                wgt[m][ww] = 1.f; // sigmoid weights: the waves' sums simply add
             L += wgt[m][ww] * ml_part[((ww * MAPS + m) * 16 + row) * 2 + 1];
         }
         if (ks > 1)
@@ -273,9 +352,10 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
         }
         else
         {
+            const float fin = finish_factor(p, h, M, L);
 #pragma unroll
             for (int ww = 0; ww < NW; ++ww)
-                wgt[m][ww] /= L;
+                wgt[m][ww] *= fin;
         }
     }
     constexpr int CPT = (V + TPR - 1) / TPR;
@@ -335,6 +415,7 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     }
     if (r0 + row < count)
     {
+        mul *= out_gate_of(p, first + r0 + row, h);
         uint16_t* out = reinterpret_cast<uint16_t*>(p.out) + ((int64_t) (first + r0 + row) * p.heads + h) * V;
 #pragma unroll
         for (int c = 0; c < CPT; ++c)
@@ -370,9 +451,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
     const int g = h / (p.heads / p.kv_heads);
     const int page = p.page;
     const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
-    constexpr float LOG2E = 1.4426950408889634f;
-    const float scale2 = p.scale * LOG2E, cap2 = p.softcap > 0.f ? p.softcap * LOG2E : 0.f;
-    const float cap_arg = p.softcap > 0.f ? p.scale / p.softcap * 2.f * LOG2E : 0.f;
+    const HeadMods hm = head_mods(p, h);
     const uint16_t* kp = reinterpret_cast<const uint16_t*>(p.k_pool);
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.v_pool);
 
@@ -380,6 +459,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
     const bool wave_rows = r0 < count; // wave-uniform
     const int qrow = r0 + col < count ? r0 + col : count - 1;
     const int qpos = pos0 + qrow;
+    const int klo = first_visible(p, qpos);
     bf16x8 qf[MAPS][DK];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m)
@@ -391,6 +471,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
     const int nblk = (pos0 + wg_last) / 32 + 1;
     const int my_last = r0 + 15 < count ? r0 + 15 : count - 1;
     const int my_blk = wave_rows ? (pos0 + my_last) / 32 : -1; // the wave's last block that holds a visible key
+    // ... and its first, and the workgroup's first (a window or a chunk hides everything before it)
+    const int my_lo = wave_rows ? first_visible(p, pos0 + r0) / 32 : 0, klo_last = wave_rows ? first_visible(p, pos0 + my_last) : 0;
+    const int wg_lo = first_visible(p, pos0 + tile * 64) / 32;
 
     float m_run[MAPS], l_run[MAPS];
     f32x4 acc[MAPS][VT];
@@ -406,7 +489,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
 
     uint4 kr[KPT], vr[VPT];
     // the page id of a block is fetched one block before its rows are requested: one memory latency per block, not two in a row
-    int blk_next = table[0];
+    int blk_next = table[wg_lo * 32 / page];
     auto request = [&](int kb) {
         const int key0 = kb * 32;
         const int blk = blk_next, off = key0 % page;
@@ -430,8 +513,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
                 vr[i] = *reinterpret_cast<const uint4*>(vp + (((int64_t) blk * p.kv_heads + g) * V + idx / 4) * page + off + (idx % 4) * 8);
         }
     };
-    request(0);
-    for (int kb = 0; kb < nblk; ++kb)
+    request(wg_lo);
+    for (int kb = wg_lo; kb < nblk; ++kb)
     {
 #pragma unroll
         for (int i = 0; i < KPT; ++i)
@@ -450,11 +533,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
         __syncthreads();
         if (kb + 1 < nblk)
             request(kb + 1);
-        if (kb <= my_blk)
+        if (kb <= my_blk && kb >= my_lo)
         {
             const int key0 = kb * 32;
             uint4 pf[MAPS];
-            const bool masked = key0 + 31 > pos0 + r0; // wave-uniform
+            const bool masked = key0 + 31 > pos0 + r0 || key0 < klo_last; // wave-uniform
 #pragma unroll
             for (int m = 0; m < MAPS; ++m)
             {
@@ -469,7 +552,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
                             as_bf16x8(*reinterpret_cast<const uint4*>(k_s + (m * 32 + t * 16 + col) * KP + (ks * 32 + 8 * g4) * 2)), qf[m][ks], s[t],
                             0, 0, 0);
                 }
-                pf[m] = softmax_block<VT>(s, m_run[m], l_run[m], acc[m], scale2, cap2, cap_arg, masked, key0 + 4 * g4, qpos);
+                pf[m] = softmax_block<VT>(s, m_run[m], l_run[m], acc[m], hm, masked, key0 + 4 * g4, qpos, klo);
             }
 #pragma unroll
             for (int ct = 0; ct < VT; ++ct)
@@ -491,7 +574,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
     float inv[MAPS];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m)
-        inv[m] = 1.f / l_run[m];
+        inv[m] = finish_factor(p, h, m_run[m], l_run[m]);
     float ss = 0.f;
 #pragma unroll
     for (int ct = 0; ct < VT; ++ct)
@@ -513,6 +596,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
     }
     if (r0 + col < count)
     {
+        mul *= out_gate_of(p, first + r0 + col, h);
         uint16_t* out = reinterpret_cast<uint16_t*>(p.out) + ((int64_t) (first + r0 + col) * p.heads + h) * V + 4 * g4;
 #pragma unroll
         for (int ct = 0; ct < VT; ++ct)
@@ -542,15 +626,16 @@ __global__ __launch_bounds__(64) void attn_split_merge_kernel(const StackAttnPar
     {
         const bool mine = owner && lane % MAPS == m;
         const float M = wave_max(mine ? pm : -INFINITY);
-        const float e_ = mine && pm != -INFINITY ? __builtin_amdgcn_exp2f(pm - M) : 0.f;
-        const float L = wave_sum(e_ * pl);
+        const float e_ = p.weights == WEIGHTS_SIGMOID ? 1.f : (mine && pm != -INFINITY ? __builtin_amdgcn_exp2f(pm - M) : 0.f);
+        const float L = wave_sum(mine ? e_ * pl : 0.f);
         if (mine)
-            wl = e_ / L;
+            wl = e_ * finish_factor(p, h, M, L);
     }
-    float o[2], ss = 0.f; // vdim <= 128: two channels per lane
-    float a[2][MAPS];
+    constexpr int MC = 4; // vdim <= 256: four channels per lane
+    float o[MC], ss = 0.f;
+    float a[MC][MAPS];
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < MC; ++c)
 #pragma unroll
         for (int m = 0; m < MAPS; ++m)
             a[c][m] = 0.f;
@@ -561,13 +646,13 @@ __global__ __launch_bounds__(64) void attn_split_merge_kernel(const StackAttnPar
         if (i < ks * MAPS) // wave-uniform
         {
 #pragma unroll
-            for (int c = 0; c < 2; ++c)
+            for (int c = 0; c < MC; ++c)
                 if (lane + c * 64 < V)
                     a[c][i % MAPS] += wgt * base[i * (V + 2) + lane + c * 64];
         }
     }
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < MC; ++c)
     {
         o[c] = 0.f;
         if (lane + c * 64 < V)
@@ -579,9 +664,10 @@ __global__ __launch_bounds__(64) void attn_split_merge_kernel(const StackAttnPar
     float mul = 1.f;
     if (p.head_norm)
         mul = p.out_scale / sqrtf(wave_sum(ss) / (float) V + p.eps);
+    mul *= out_gate_of(p, t, h);
     uint16_t* out = reinterpret_cast<uint16_t*>(p.out) + ((int64_t) t * p.heads + h) * V;
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < MC; ++c)
         if (lane + c * 64 < V)
             out[lane + c * 64] = f2bf(o[c] * mul);
 }
@@ -612,7 +698,9 @@ int launch_tile(const StackAttnParams& p, hipStream_t stream)
         int ks = 1;
         if (p.split_ws && p.max_count <= 16 && p.tokens <= kSplitRows)
         {
-            const int nblk = (p.max_context + 31) / 32;
+            // a window or a chunk bounds the keys a row walks
+            const int span = p.mask == MASK_CAUSAL ? p.max_context : std::min(p.max_context, p.mask_size + 31);
+            const int nblk = (span + 31) / 32;
             ks = std::min(kMaxSplits, (nblk + 2 * NW - 1) / (2 * NW));
         }
         const dim3 grid(ks > 1 ? ks : (small_rows + 15) / 16, p.entries, p.heads);
@@ -641,6 +729,16 @@ int launch_tile_v(const StackAttnParams& p, hipStream_t stream)
     }
 }
 
+// one shared key/value head of dim = latent + rotated part, vdim = latent (latent attention in absorbed form)
+int launch_tile_latent(const StackAttnParams& p, hipStream_t stream)
+{
+    if (p.dim == 160 && p.vdim == 128)
+        return launch_tile<1, 5, 8>(p, stream);
+    if (p.dim == 320 && p.vdim == 256)
+        return launch_tile<1, 10, 16>(p, stream);
+    return 1;
+}
+
 template <int MAPS>
 int launch_tile_d(const StackAttnParams& p, hipStream_t stream)
 {
@@ -664,9 +762,9 @@ size_t stack_attn_workspace_floats(int32_t heads, int32_t maps, int32_t vdim)
 // the tile kernel's shapes: bfloat16, dim 32 / 64 / 128, vdim 32 / 64 / 128, pages of a multiple of 32 keys
 bool stack_attention_tiled(const StackAttnParams& p)
 {
-    return p.dtype == DT_BF16 && (p.dim == 32 || p.dim == 64 || p.dim == 128) && (p.vdim == 32 || p.vdim == 64 || p.vdim == 128)
-        && !p.temp && !p.slope && !p.log_r1 && p.mask == MASK_CAUSAL && p.weights == WEIGHTS_SOFTMAX && !p.sink && !p.out_gate
-        && p.page % 32 == 0 && p.max_count > 0 && p.entries > 0 && !(reinterpret_cast<uintptr_t>(p.q) & 15)
+    const bool std_shape = (p.dim == 32 || p.dim == 64 || p.dim == 128) && (p.vdim == 32 || p.vdim == 64 || p.vdim == 128);
+    const bool latent_shape = p.maps == 1 && p.kv_heads == 1 && ((p.dim == 160 && p.vdim == 128) || (p.dim == 320 && p.vdim == 256));
+    return p.dtype == DT_BF16 && (std_shape || latent_shape) && p.page % 32 == 0 && p.max_count > 0 && p.entries > 0 && !(reinterpret_cast<uintptr_t>(p.q) & 15)
         && !(reinterpret_cast<uintptr_t>(p.k_pool) & 15) && !(reinterpret_cast<uintptr_t>(p.v_pool) & 7);
 }
 
@@ -676,7 +774,9 @@ int launch_stack_attention(const StackAttnParams& p, hipStream_t stream)
         return 0;
     if (p.heads >= 1 && p.kv_heads >= 1 && p.heads % p.kv_heads == 0 && stack_attention_tiled(p))
     {
-        const int rc = p.maps == 2 ? launch_tile_d<2>(p, stream) : (p.maps == 1 ? launch_tile_d<1>(p, stream) : 1);
+        int rc = p.maps == 2 ? launch_tile_d<2>(p, stream) : (p.maps == 1 ? launch_tile_d<1>(p, stream) : 1);
+        if (rc == 1 && p.maps == 1)
+            rc = launch_tile_latent(p, stream);
         if (rc <= 0)
             return rc;
     }

@@ -64,7 +64,7 @@ def generate(model_dir, max_output_len, dtype='bfloat16', input_file=None, end_i
         np.save(output_npy, np.array([r + [pad_id] * (width - len(r)) for r in rows], np.int32))
     for r, p in zip(rows, prompts):
         print('Output ids:', r[len(p):])
-    print(f'tolenex-run ({sum(len(o) for o in outs)} tokens in {dt:.3f} sec)')
+    print(f'{model.architecture.lower()}-run ({sum(len(o) for o in outs)} tokens in {dt:.3f} sec)')
     return rows
 
 
