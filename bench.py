@@ -62,9 +62,11 @@ def parse():
     ap.add_argument('--parity-prompts', type=int, default=8, help='seeded prompts of the accuracy report')
     ap.add_argument('--cpu-tokens', type=int, default=0, help='CPU-baseline decode steps (0 = sized to ~20 s)')
     ap.add_argument('--cpu-threads', type=int, default=0)
-    ap.add_argument('--design', default='llama', choices=['llama', 'tolenex'],
+    ap.add_argument('--design', default='llama', choices=['llama', 'tolenex', 'vetipel'],
                     help="tolenex: a side report instead of the headline workload - prefill and decode throughput of the Tolenex design "
-                         "(bfloat16, ragged stack engine) at layer sizes of real models, beside LLaMA fp16 at equal size")
+                         "(bfloat16, ragged stack engine) at layer sizes of real models, beside LLaMA fp16 at equal size; "
+                         "vetipel: the same report for the Vetipel design, beside Tolenex (the closest model: same engine, bfloat16) and "
+                         "LLaMA fp16 at equal size")
     ap.add_argument('--design-sizes', default='2048,4096', help='--design tolenex: comma list of model widths')
     ap.add_argument('--design-no-llama', action='store_true', help='--design tolenex: skip the LLaMA side (kernel traces of the new design alone)')
     ap.add_argument('--design-layers', type=int, default=4, help='--design tolenex: layers of both models')
@@ -589,6 +591,50 @@ def tolenex_config(width, layers, vocab=32000):
             'layers': [rec if i % 4 == 2 else attn for i in range(layers)]}
 
 
+def vetipel_config(width, layers, vocab=32000):
+    """A Vetipel configuration with the layer sizes of a LLaMA-like model of this width: heads of 128, four query heads per key /
+    value head, windows and chunks of 512 tokens, a latent of 256 + 64 rotated dimensions under heads of 64 + 64 query / key and 128
+    value dimensions, two residual streams, feed-forward 2.6875 x width.  Layers cycle window / latent / chunk / window."""
+    heads = width // 128
+    ff = {'ff': int(width * 2.6875), 'kind': 'dense'}
+    gq = {'heads': heads, 'kv_heads': max(heads // 4, 1), 'dim': 128, 'vdim': 128, 'scale': 128 ** -0.5, 'mask': {'size': 512}}
+    lat = {'heads': heads, 'dim': 64, 'rot_dim': 64, 'vdim': 128, 'kv_rank': 256, 'scale': 128 ** -0.5, 'rot': {'dims': 64, 'base': 500000.0}}
+    kinds = [('attention', gq), ('latent_attention', lat), ('attention_2', gq), ('attention', gq)]
+    return {'architecture': 'Vetipel', 'vocab': vocab, 'width': width, 'embedding': {'scale': 8.0}, 'norm': {'eps': 1e-6}, 'streams': 2,
+            'layers': [{'type': kinds[i % 4][0], 'mixer': dict(kinds[i % 4][1]), 'mlp': dict(ff)} for i in range(layers)]}
+
+
+def time_stack_model(torch, model, vocab, S, K, W, tag, row):
+    """Prefill (one step of S prompt tokens) and decode (single tokens at context S, 1 and 4 sequences per step) of a stack-engine
+    model in bfloat16 through RaggedGenerationSession.step; wall clock around synchronised calls."""
+    from tensorrt_llm.runtime import RaggedGenerationSession
+    sess = RaggedGenerationSession(model, dtype='bfloat16', max_tokens=4 * (S + 2 * K + 2 * W + 64), max_sequences=4, max_batch_tokens=S)
+    prompt = np.random.default_rng(0).integers(0, vocab, S).tolist()
+    row[f'{tag}_weight_bytes'] = sess.engine.weight_bytes()
+    sess.step([('warm', prompt, [S - 1])], end=['warm'])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    sess.step([('p', prompt, [S - 1])])
+    t_prefill = time.perf_counter() - t0
+    row[f'{tag}_prefill_ms'] = t_prefill * 1e3
+    row[f'{tag}_prefill_tokens_per_s'] = S / t_prefill
+    for batch in (1, 4):
+        ids = ['p'] + [f'q{b}' for b in range(1, batch)]
+        for rid in ids[1:]:
+            sess.step([(rid, prompt, [])])
+        for _ in range(W):
+            sess.step([(rid, [7], [0]) for rid in ids], return_logits=False)
+        t0 = time.perf_counter()
+        for _ in range(K):
+            sess.step([(rid, [7], [0]) for rid in ids], return_logits=False)
+        dt = time.perf_counter() - t0
+        row[f'{tag}_decode_b{batch}_tokens_per_s'] = batch * K / dt
+        row[f'{tag}_decode_b{batch}_ms_per_step'] = dt * 1e3 / K
+        ctx = sess.length_of('p')
+        row[f'{tag}_decode_b{batch}_hbm_fraction'] = sess.engine.step_bytes(batch, batch * ctx, batch) / (dt / K) / 8e12
+    return prompt
+
+
 def tolenex_report(torch, args, dev):
     """Prefill (one step of S prompt tokens) and decode (single tokens at context S, 1 and 4 sequences per step) of Tolenex in
     bfloat16 through RaggedGenerationSession.step, and the same two phases of LLaMA fp16 (the closest model the framework has: same
@@ -602,34 +648,15 @@ def tolenex_report(torch, args, dev):
     for width in [int(v) for v in args.design_sizes.split(',')]:
         L = args.design_layers
         cfg = tolenex_config(width, L)
+        row = dict(width=width, layers=L, context=S)
+        if args.design == 'vetipel':
+            from tensorrt_llm.models import VetipelForCausalLM
+            vcfg = vetipel_config(width, L)
+            time_stack_model(torch, VetipelForCausalLM.from_random(vcfg, seed=1), vcfg['vocab'], S, K, W, 'vetipel', row)
         model = TolenexForCausalLM.from_random(cfg, seed=1)
-        sess = RaggedGenerationSession(model, dtype='bfloat16', max_tokens=4 * (S + 2 * K + 2 * W + 64), max_sequences=4,
-                                       max_batch_tokens=S)
-        rng = np.random.default_rng(0)
-        prompt = rng.integers(0, cfg['vocab'], S).tolist()
-        row = dict(width=width, layers=L, context=S, weight_bytes=sess.engine.weight_bytes())
-        sess.step([('warm', prompt, [S - 1])], end=['warm'])
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        sess.step([('p', prompt, [S - 1])])
-        t_prefill = time.perf_counter() - t0
-        row['tolenex_prefill_ms'] = t_prefill * 1e3
-        row['tolenex_prefill_tokens_per_s'] = S / t_prefill
-        for batch in (1, 4):
-            ids = ['p'] + [f'q{b}' for b in range(1, batch)]
-            for rid in ids[1:]:
-                sess.step([(rid, prompt, [])])
-            for _ in range(W):
-                sess.step([(rid, [7], [0]) for rid in ids], return_logits=False)
-            t0 = time.perf_counter()
-            for _ in range(K):
-                sess.step([(rid, [7], [0]) for rid in ids], return_logits=False)
-            dt = time.perf_counter() - t0
-            row[f'tolenex_decode_b{batch}_tokens_per_s'] = batch * K / dt
-            row[f'tolenex_decode_b{batch}_ms_per_step'] = dt * 1e3 / K
-            ctx = sess.length_of('p')
-            row[f'tolenex_decode_b{batch}_hbm_fraction'] = sess.engine.step_bytes(batch, batch * ctx, batch) / (dt / K) / 8e12
-        del sess, model
+        prompt = time_stack_model(torch, model, cfg['vocab'], S, K, W, 'tolenex', row)
+        row['weight_bytes'] = row['tolenex_weight_bytes']
+        del model
         if args.design_no_llama:
             rows.append({k: (round(v, 3) if isinstance(v, float) else v) for k, v in row.items()})
             continue
@@ -666,7 +693,7 @@ def tolenex_report(torch, args, dev):
         ls.close()
         rows.append({k: (round(v, 3) if isinstance(v, float) else v) for k, v in row.items()})
         print(f'[bench] {rows[-1]}', file=sys.stderr, flush=True)
-    print(json.dumps({'metric': 'tolenex_side_report', 'dtype': 'bf16 (Tolenex) / fp16 (LLaMA)', 'data': 'synthetic', 'n_gpus': 1,
+    print(json.dumps({'metric': f'{args.design}_side_report', 'dtype': 'bf16 (stack engine designs) / fp16 (LLaMA)', 'data': 'synthetic', 'n_gpus': 1,
                       'steps': K, 'warmup': W, 'sizes': rows}))
 
 
@@ -703,9 +730,9 @@ def main():
         local = 0
     torch.cuda.set_device(local)
     dev = torch.device('cuda', local)
-    if args.design == 'tolenex':
+    if args.design in ('tolenex', 'vetipel'):
         if world != 1:
-            raise SystemExit('--design tolenex is a one-GPU report')
+            raise SystemExit(f'--design {args.design} is a one-GPU report')
         return tolenex_report(torch, args, dev)
     dist = None
     if world > 1:
