@@ -69,6 +69,7 @@ def parse():
                          "LLaMA fp16 at equal size")
     ap.add_argument('--design-sizes', default='2048,4096', help='--design tolenex: comma list of model widths')
     ap.add_argument('--design-no-llama', action='store_true', help='--design tolenex: skip the LLaMA side (kernel traces of the new design alone)')
+    ap.add_argument('--design-alone', action='store_true', help='--design vetipel: time that design only (kernel traces without its neighbours)')
     ap.add_argument('--design-layers', type=int, default=4, help='--design tolenex: layers of both models')
     ap.add_argument('--cpu-sweep', default='', help='debug: comma list of thread counts to try (stderr)')
     return ap.parse_args()
@@ -653,6 +654,10 @@ def tolenex_report(torch, args, dev):
             from tensorrt_llm.models import VetipelForCausalLM
             vcfg = vetipel_config(width, L)
             time_stack_model(torch, VetipelForCausalLM.from_random(vcfg, seed=1), vcfg['vocab'], S, K, W, 'vetipel', row)
+            if args.design_alone:
+                rows.append({k: (round(v, 3) if isinstance(v, float) else v) for k, v in row.items()})
+                print(f'[bench] {rows[-1]}', file=sys.stderr, flush=True)
+                continue
         model = TolenexForCausalLM.from_random(cfg, seed=1)
         prompt = time_stack_model(torch, model, cfg['vocab'], S, K, W, 'tolenex', row)
         row['weight_bytes'] = row['tolenex_weight_bytes']

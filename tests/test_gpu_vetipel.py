@@ -151,6 +151,21 @@ def test_requests_of_very_unequal_length_decode_side_by_side(dtype):
         check(got[rid], O.logits(toks, as_f64(w), cfg), tol_of(dtype), rid)
 
 
+@pytest.mark.parametrize('heads', [8, 20, 32])
+def test_decoding_where_many_heads_share_one_key_value_head(heads):
+    """Latent attention with 8 and more heads, single decoded tokens: the tile kernel walks the shared keys once per 16 heads (a
+    head count that is not a multiple of 16 leaves part of the last tile empty), beside a request that brings a prompt portion."""
+    cfg = make_config([latent_layer(heads=heads, dim=32, rot_dim=32, vdim=32, kv_rank=128, ff=0), window_layer(ff=40)], streams=2)
+    w = random_weights(cfg, seed=23)
+    reqs = {'a': tokens_for(cfg, 140, 93), 'b': tokens_for(cfg, 45, 94)}
+    schedule = [[('a', 70)]] + [[('a', 1)]] * 30 + [[('a', 1), ('b', 1)]] * 5 + [[('a', 1), ('b', 40)]] + [[('a', 1)]] * 34
+    for dtype in ('bfloat16', 'float32'):
+        s = session_for(cfg, w, dtype)
+        got = replay(s, reqs, schedule)
+        for rid, toks in reqs.items():
+            check(got[rid], O.logits(toks, as_f64(w), cfg), tol_of(dtype), f'{dtype} {rid}')
+
+
 def test_pages_and_slots_that_are_used_again():
     """A pool of 4 pages and 2 slots serves six requests one after another and side by side: every page is written by several
     requests, and what an earlier request left in a page must never be seen through a window, a chunk or the causal mask."""

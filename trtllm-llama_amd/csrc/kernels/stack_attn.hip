@@ -187,7 +187,7 @@ __device__ __forceinline__ float out_gate_of(const StackAttnParams& p, int64_t t
 }
 
 template <int MAPS, int DK, int VT, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParams p, int below_count, int ks)
+__global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParams p, int below_count, int ks, int head_rows)
 {
     constexpr int D = DK * 32, V = VT * 16;
     extern __shared__ float lds[];
@@ -196,7 +196,10 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     // ks == 1: blockIdx.x is the entry's 16-row tile.  ks > 1 (decoding steps: every entry one tile): blockIdx.x is the key split -
     // workgroup `split` of an (entry, head) takes the key blocks split * NW + w, + ks * NW, ... and leaves an unnormalised partial
     // (max, sum, O per map and row) in split_ws; attn_split_merge_kernel finishes the rows.
-    const int e = blockIdx.y, h = blockIdx.z, r0 = ks > 1 ? 0 : blockIdx.x * 16;
+    // head_rows (a step of single decoded tokens whose heads all share ONE key/value head and have no numbers of their own): the
+    // tile's 16 rows are 16 HEADS of the entry's one token, blockIdx.z the group of heads - the keys are walked once per 16 heads
+    const int e = blockIdx.y, hbase = head_rows ? blockIdx.z * 16 : 0, h = head_rows ? hbase : blockIdx.z;
+    const int r0 = (ks > 1 || head_rows) ? 0 : blockIdx.x * 16;
     const int split = ks > 1 ? blockIdx.x : 0;
     const int count = p.ent_count[e];
     if (r0 >= count || count >= below_count) // entries of below_count rows and more are the prefill form's
@@ -211,7 +214,8 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     const uint16_t* kp = reinterpret_cast<const uint16_t*>(p.k_pool);
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.v_pool);
 
-    const int qrow = r0 + col < count ? r0 + col : count - 1;
+    const int qrow = head_rows ? 0 : (r0 + col < count ? r0 + col : count - 1);
+    const int qhead = head_rows ? (hbase + col < p.heads ? hbase + col : p.heads - 1) : h;
     const int qpos = pos0 + qrow;
     const int klo = first_visible(p, qpos);
     bf16x8 qf[MAPS][DK];
@@ -220,8 +224,8 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
 #pragma unroll
         for (int ks = 0; ks < DK; ++ks)
             qf[m][ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
-                reinterpret_cast<const uint16_t*>(p.q) + (((int64_t) (first + qrow) * p.heads + h) * MAPS + m) * D + ks * 32 + 8 * g4));
-    const int last_row = r0 + 15 < count ? r0 + 15 : count - 1;
+                reinterpret_cast<const uint16_t*>(p.q) + (((int64_t) (first + qrow) * p.heads + qhead) * MAPS + m) * D + ks * 32 + 8 * g4));
+    const int last_row = head_rows ? 0 : (r0 + 15 < count ? r0 + 15 : count - 1);
     const int nblk = (pos0 + last_row) / 32 + 1;
     // the tile's key blocks: from the one that holds the first row's first visible key; klo_last: the last row's (the largest)
     const int blk_lo = first_visible(p, pos0 + r0) / 32, klo_last = first_visible(p, pos0 + last_row);
@@ -322,6 +326,10 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     // 16 threads per row at NW = 4 (NW * 4 in general), each a strided set of channels
     constexpr int TPR = NW * 4;
     const int row = threadIdx.x / TPR, sub = threadIdx.x % TPR;
+    // where tile row `row` leaves: (packed row, head)
+    const int64_t out_t = first + (head_rows ? 0 : r0 + row);
+    const int out_h = head_rows ? hbase + row : h;
+    const bool out_ok = head_rows ? hbase + row < p.heads : r0 + row < count;
     float wgt[MAPS][NW];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m)
@@ -343,9 +351,9 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
         if (ks > 1)
         {
             // partial of this split: weights stay relative to the split's own maximum, nothing is divided yet
-            if (sub == 0 && r0 + row < count)
+            if (sub == 0 && out_ok)
             {
-                float* ws = p.split_ws + ((((int64_t) (first + row) * p.heads + h) * ks + split) * MAPS + m) * (V + 2);
+                float* ws = p.split_ws + (((out_t * p.heads + out_h) * ks + split) * MAPS + m) * (V + 2);
                 ws[V] = M;
                 ws[V + 1] = L;
             }
@@ -361,12 +369,12 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     constexpr int CPT = (V + TPR - 1) / TPR;
     if (ks > 1)
     {
-        if (r0 + row < count)
+        if (out_ok)
         {
 #pragma unroll
             for (int m = 0; m < MAPS; ++m)
             {
-                float* ws = p.split_ws + ((((int64_t) (first + row) * p.heads + h) * ks + split) * MAPS + m) * (V + 2);
+                float* ws = p.split_ws + (((out_t * p.heads + out_h) * ks + split) * MAPS + m) * (V + 2);
 #pragma unroll
                 for (int c = 0; c < CPT; ++c)
                 {
@@ -413,10 +421,10 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
             ss += __shfl_xor(ss, d, 64);
         mul = p.out_scale / sqrtf(ss / (float) V + p.eps);
     }
-    if (r0 + row < count)
+    if (out_ok)
     {
-        mul *= out_gate_of(p, first + r0 + row, h);
-        uint16_t* out = reinterpret_cast<uint16_t*>(p.out) + ((int64_t) (first + r0 + row) * p.heads + h) * V;
+        mul *= out_gate_of(p, out_t, out_h);
+        uint16_t* out = reinterpret_cast<uint16_t*>(p.out) + (out_t * p.heads + out_h) * V;
 #pragma unroll
         for (int c = 0; c < CPT; ++c)
             if (sub + c * TPR < V)
@@ -703,8 +711,13 @@ int launch_tile(const StackAttnParams& p, hipStream_t stream)
             const int nblk = (span + 31) / 32;
             ks = std::min(kMaxSplits, (nblk + 2 * NW - 1) / (2 * NW));
         }
-        const dim3 grid(ks > 1 ? ks : (small_rows + 15) / 16, p.entries, p.heads);
-        hipLaunchKernelGGL((attn_tile_kernel<MAPS, DK, VT, NW>), grid, dim3(NW * 64), lds, stream, p, PREFILL_ROWS, ks);
+        // single decoded tokens whose heads share one key/value head and carry no per-head numbers: 16 heads are the tile's rows
+        const int head_rows = (p.max_count == 1 && p.kv_heads == 1 && MAPS == 1 && p.heads >= 8 && !p.temp && !p.slope && !p.log_r1 && !p.sink
+                                  && !p.wbias && !p.head_norm)
+            ? 1
+            : 0;
+        const dim3 grid(ks > 1 ? ks : (small_rows + 15) / 16, p.entries, head_rows ? (p.heads + 15) / 16 : p.heads);
+        hipLaunchKernelGGL((attn_tile_kernel<MAPS, DK, VT, NW>), grid, dim3(NW * 64), lds, stream, p, PREFILL_ROWS, ks, head_rows);
         if (ks > 1)
             hipLaunchKernelGGL((attn_split_merge_kernel<MAPS>), dim3(p.tokens, p.heads), dim3(64), 0, stream, p, ks, PREFILL_ROWS);
     }

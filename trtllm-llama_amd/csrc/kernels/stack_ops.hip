@@ -827,6 +827,113 @@ int launch_stack_embed(float* x, float* keep, const int32_t* ids, const void* ta
     return launched("stack_embed");
 }
 
+// The form for rows of a multiple of 4 up to HV_K * 4096 elements: up to 1024 threads, a thread owns HV_K float4 columns of every
+// stream and has ALL of them in flight before its first store (the streams are read and written through the same pointer, so in
+// a loop every store would fence the loads behind it); the combined row stays in registers.
+constexpr int HV_K = 2;
+
+template <int DT, int SM>
+__global__ __launch_bounds__(1024) void hyper_norm_vec_kernel(const StackHyperParams p)
+{
+    __shared__ float red[32];
+    const int t = blockIdx.x, tid = threadIdx.x, S = p.streams, W4 = p.width >> 2, NT = blockDim.x;
+    float4 xs[HV_K][SM], yv[HV_K], u[HV_K];
+#pragma unroll
+    for (int k = 0; k < HV_K; ++k)
+    {
+        const int c4 = tid + k * NT;
+        yv[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int s = 0; s < SM; ++s)
+            xs[k][s] = (s < S && c4 < W4) ? reinterpret_cast<const float4*>(p.x + s * p.stream_stride + (int64_t) t * p.width)[c4]
+                                          : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (p.y && c4 < W4)
+            yv[k] = reinterpret_cast<const float4*>(p.y + (int64_t) t * p.width)[c4];
+    }
+    float cm[SM][SM], co[SM], ci[SM];
+#pragma unroll
+    for (int a = 0; a < SM; ++a)
+    {
+        co[a] = (p.y && a < S) ? p.out[a] : 0.f;
+        ci[a] = a < S ? (p.in ? p.in[a] : 1.f) : 0.f;
+#pragma unroll
+        for (int b = 0; b < SM; ++b)
+            cm[a][b] = (p.y && a < S && b < S) ? p.mix[a * S + b] : 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < HV_K; ++k)
+    {
+        const int c4 = tid + k * NT;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int to = 0; to < SM; ++to)
+        {
+            float4 n = xs[k][to];
+            if (p.y)
+            {
+                n = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int s = 0; s < SM; ++s)
+                {
+                    n.x = fmaf(cm[s][to], xs[k][s].x, n.x);
+                    n.y = fmaf(cm[s][to], xs[k][s].y, n.y);
+                    n.z = fmaf(cm[s][to], xs[k][s].z, n.z);
+                    n.w = fmaf(cm[s][to], xs[k][s].w, n.w);
+                }
+                n.x = fmaf(co[to], yv[k].x, n.x);
+                n.y = fmaf(co[to], yv[k].y, n.y);
+                n.z = fmaf(co[to], yv[k].z, n.z);
+                n.w = fmaf(co[to], yv[k].w, n.w);
+                if (to < S && c4 < W4)
+                    reinterpret_cast<float4*>(p.x + to * p.stream_stride + (int64_t) t * p.width)[c4] = n;
+            }
+            acc.x = fmaf(ci[to], n.x, acc.x);
+            acc.y = fmaf(ci[to], n.y, acc.y);
+            acc.z = fmaf(ci[to], n.z, acc.z);
+            acc.w = fmaf(ci[to], n.w, acc.w);
+        }
+        u[k] = acc;
+        if (p.sum_out && c4 < W4)
+            reinterpret_cast<float4*>(p.sum_out + (int64_t) t * p.width)[c4] = acc;
+        ss += acc.x * acc.x + acc.y * acc.y + acc.z * acc.z + acc.w * acc.w;
+    }
+    if (!p.h)
+        return;
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float) p.width + p.eps);
+#pragma unroll
+    for (int k = 0; k < HV_K; ++k)
+    {
+        const int c4 = tid + k * NT;
+        if (c4 < W4)
+        {
+            const float4 w = reinterpret_cast<const float4*>(p.w)[c4];
+            const int64_t o = (int64_t) t * p.width + 4 * c4;
+            if (DT == DT_BF16)
+                *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.h) + o)
+                    = make_uint2((uint32_t) f2bf(u[k].x * inv * w.x) | ((uint32_t) f2bf(u[k].y * inv * w.y) << 16),
+                        (uint32_t) f2bf(u[k].z * inv * w.z) | ((uint32_t) f2bf(u[k].w * inv * w.w) << 16));
+            else
+                *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.h) + o)
+                    = make_float4(u[k].x * inv * w.x, u[k].y * inv * w.y, u[k].z * inv * w.z, u[k].w * inv * w.w);
+        }
+    }
+}
+
+template <int DT>
+static void launch_hyper_vec(const StackHyperParams& p, int nt, hipStream_t stream)
+{
+    if (p.streams <= 1)
+        hipLaunchKernelGGL((hyper_norm_vec_kernel<DT, 1>), dim3(p.tokens), dim3(nt), 0, stream, p);
+    else if (p.streams <= 2)
+        hipLaunchKernelGGL((hyper_norm_vec_kernel<DT, 2>), dim3(p.tokens), dim3(nt), 0, stream, p);
+    else if (p.streams <= 4)
+        hipLaunchKernelGGL((hyper_norm_vec_kernel<DT, 4>), dim3(p.tokens), dim3(nt), 0, stream, p);
+    else
+        hipLaunchKernelGGL((hyper_norm_vec_kernel<DT, 8>), dim3(p.tokens), dim3(nt), 0, stream, p);
+}
+
 int launch_stack_hyper_norm(const StackHyperParams& p, hipStream_t stream)
 {
     if (p.tokens <= 0)
@@ -837,6 +944,17 @@ int launch_stack_hyper_norm(const StackHyperParams& p, hipStream_t stream)
     {
         set_error("stack_hyper_norm: %d streams (1 .. %d) of width %d, or a missing operand", p.streams, HY_MAXS, p.width);
         return -1;
+    }
+    const bool al16 = !(reinterpret_cast<uintptr_t>(p.x) & 15) && !(reinterpret_cast<uintptr_t>(p.y) & 15) && !(reinterpret_cast<uintptr_t>(p.h) & 15)
+        && !(reinterpret_cast<uintptr_t>(p.w) & 15) && !(reinterpret_cast<uintptr_t>(p.sum_out) & 15) && p.stream_stride % 4 == 0;
+    if (p.width % 4 == 0 && p.width <= HV_K * 4096 && al16)
+    {
+        const int nt = std::min(1024, (p.width / 4 + 63) / 64 * 64);
+        if (p.dtype == DT_BF16)
+            launch_hyper_vec<DT_BF16>(p, nt, stream);
+        else
+            launch_hyper_vec<DT_FLOAT>(p, nt, stream);
+        return launched("stack_hyper_norm");
     }
     const size_t lds = sizeof(float) * (size_t) p.width;
     if (lds > 64 * 1024)
