@@ -65,8 +65,16 @@ __device__ __forceinline__ void wait_vmcnt()
 // third of every compute wave's issue time; loaders (the shape's 160 VGPRs leave room for a third wave per SIMD) take that
 // over and run the ring's look-ahead.
 template <int WT, int WM, int WN, int MT, int NT, int KG, int BKB, int S, int LW = 0>
-__global__ __launch_bounds__(64 * (WM * WN * KG + LW)) void gemm_glds_kernel(const GemmParams p)
+__global__ __launch_bounds__(64 * (WM * WN * KG + LW)) void gemm_glds_kernel(const GemmParams p_in)
 {
+    GemmParams p = p_in;
+    if constexpr (WT == W_BF16)
+    {
+        // a batch of independent products of one shape (the stack engine's per-head products): blockIdx.y picks the operands
+        p.a = reinterpret_cast<const char*>(p.a) + (int64_t) blockIdx.y * p.batch_a;
+        p.w = reinterpret_cast<const char*>(p.w) + (int64_t) blockIdx.y * p.batch_w;
+        p.c = reinterpret_cast<char*>(p.c) + (int64_t) blockIdx.y * p.batch_c;
+    }
     constexpr bool SQ = WT == W_INT8_SQ;
     constexpr int ES = SQ ? 1 : 2; // bytes per A / W element
     constexpr int NWC = WM * WN * KG;             // compute waves: KG groups of WM x WN waves split the k-steps of every stage
@@ -501,7 +509,7 @@ int launch_cfg(const GemmParams& p, hipStream_t stream)
     auto kfn = gemm_glds_kernel<WT, WM, WN, MT, NT, KG, BKB, S, LW>;
     launch_util::ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), smem);
     const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-    hipLaunchKernelGGL(kfn, dim3(tiles), dim3(64 * (WM * WN * KG + LW)), smem, stream, p);
+    hipLaunchKernelGGL(kfn, dim3(tiles, WT == W_BF16 && p.batch > 1 ? p.batch : 1), dim3(64 * (WM * WN * KG + LW)), smem, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess)
     {

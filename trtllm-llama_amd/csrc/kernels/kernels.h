@@ -362,6 +362,10 @@ struct GemmParams
     // W_BF16 only, without resid: + bias[n] (fp32 [N]) on the accumulator; act 1: max(v, 0)^2 of the value rounded to the output type
     const float* bias = nullptr;
     int32_t act = 0;
+    // W_BF16 on the LDS-DMA tiles only: `batch` products of this shape in one launch, operands of product b at a + b * batch_a bytes,
+    // w + b * batch_w, c + b * batch_c (no resid / residual)
+    int32_t batch = 1;
+    int64_t batch_a = 0, batch_w = 0, batch_c = 0;
     // microbench hook (tllm_gemm_set_clock_probe), set by the launchers only: 2 x uint64 per workgroup {shader cycles, 100 MHz ticks}
     void* clock_probe = nullptr;
     // split-K-2 forms of gemm_sqp.hip (r06), set by the launcher only: per tile two slabs of AH x BN accumulators + two flag words

@@ -212,7 +212,7 @@ int launch_glds_bf16(const GemmParams& g, hipStream_t stream)
     int pick = 0;
     for (const Shape& sh : shapes)
     {
-        const int64_t tiles = (int64_t) ((g.M + sh.bm - 1) / sh.bm) * ((g.N + sh.bn - 1) / sh.bn);
+        const int64_t tiles = (int64_t) ((g.M + sh.bm - 1) / sh.bm) * ((g.N + sh.bn - 1) / sh.bn) * (g.batch > 1 ? g.batch : 1);
         const double cost = (double) ((tiles + cus - 1) / cus) * sh.bm * sh.bn * sh.f;
         if (cost < best)
         {
@@ -271,9 +271,11 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
     }
     if (aligned)
     {
-        // the MFMA tile kernels take one product per launch: a batch is a sequence of launches
+        // the LDS-DMA tiles take a batch in one launch (blockIdx.y); the register-staged tiles one product per launch
+        const bool glds = p.M >= 32 && p.K % 64 == 0;
+        const int launches = glds ? 1 : p.batch;
         int rc = 0;
-        for (int b = 0; b < p.batch && rc == 0; ++b)
+        for (int b = 0; b < launches && rc == 0; ++b)
         {
             GemmParams g;
             g.wtype = W_BF16;
@@ -294,8 +296,14 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
             g.gate_bias = p.gate_bias;
             g.bias = p.bias;
             g.act = p.act;
-            if (p.M >= 32 && p.K % 64 == 0)
+            if (glds)
+            {
+                g.batch = p.batch;
+                g.batch_a = p.stride_a * 2;
+                g.batch_w = p.stride_w * 2;
+                g.batch_c = p.stride_c * (p.out_f32 ? 4 : 2);
                 rc = launch_glds_bf16(g, stream);
+            }
             else
                 rc = launch_gemm_mfma(g, stream);
         }
