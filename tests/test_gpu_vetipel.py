@@ -60,6 +60,7 @@ MECHANISMS = {
     'latent_no_rotated_part_turns': make_config([latent_layer(dims=0)]),
     'latent_many_heads': make_config([latent_layer(heads=7, dim=6, rot_dim=2, vdim=10, kv_rank=18)], width=72),
     'latent_tile_160_128': make_config([TILED[1]]),
+    'latent_tile_320_256': make_config([latent_layer(heads=2, dim=16, rot_dim=64, vdim=16, kv_rank=256, ff=0)]),
     'chunk_alone': make_config([chunk_layer()]),
     'chunk_of_one': make_config([chunk_layer(size=1, ff=40)]),
     'chunk_a_page': make_config([chunk_layer(size=64)]),
@@ -71,6 +72,7 @@ MECHANISMS = {
     'five_streams': make_config(FULL[:3], streams=5),
     'whole_stack': make_config(FULL, emb_scale=1.0, eps=3e-6),
     'tiled_stack': make_config(TILED, streams=2),
+    'width_that_is_no_multiple_of_four': make_config([window_layer(ff=30), latent_layer(ff=0), chunk_layer(ff=22)], width=70, vocab=131, streams=2),
     'wide_values': make_config([window_layer(heads=2, kv_heads=1, dim=8, vdim=160, size=20)]),
 }
 
@@ -164,6 +166,22 @@ def test_decoding_where_many_heads_share_one_key_value_head(heads):
         got = replay(s, reqs, schedule)
         for rid, toks in reqs.items():
             check(got[rid], O.logits(toks, as_f64(w), cfg), tol_of(dtype), f'{dtype} {rid}')
+
+
+@pytest.mark.parametrize('wide', ['0', '1'])
+def test_both_prefill_forms_of_long_head_rows(wide, monkeypatch):
+    """Heads of 160 and more dimensions have two staged prompt forms (64 or 128 rows per workgroup, chosen by how many workgroups
+    the step makes); both are forced here, on whole prompts, portions that end inside a tile, and mixed steps."""
+    monkeypatch.setenv('TLLM_STACK_WIDE_PREFILL', wide)
+    cfg = make_config([latent_layer(heads=3, dim=32, rot_dim=32, vdim=32, kv_rank=128, ff=0),
+                       latent_layer(heads=2, dim=16, rot_dim=64, vdim=16, kv_rank=256, ff=40)], streams=2)
+    w = random_weights(cfg, seed=25)
+    reqs = {'a': tokens_for(cfg, 300, 95), 'b': tokens_for(cfg, 171, 96)}
+    schedule = [[('a', 129), ('b', 33)], [('a', 1), ('b', 130)], [('a', 150), ('b', 1)], [('a', 20), ('b', 7)]]
+    s = session_for(cfg, w, 'bfloat16')
+    got = replay(s, reqs, schedule)
+    for rid, toks in reqs.items():
+        check(got[rid], O.logits(toks, as_f64(w), cfg), BF16_TOL, rid)
 
 
 def test_pages_and_slots_that_are_used_again():

@@ -613,6 +613,174 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
     }
 }
 
+// attn_prefill_wide_kernel: the staged form for one map and long rows (dim of 160 and more), where the fragment reads out of LDS, not
+// the matrix pipe, bound attn_prefill_kernel: a wave owns TWO 16-row tiles (a workgroup 128 rows) and every K and V^T fragment it reads
+// from LDS feeds both, which halves the LDS traffic per score.  Same staging, same products, same finish.
+template <int DK, int VT>
+__global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const StackAttnParams p, int min_count)
+{
+    constexpr int RT = 2, ROWS = 64 * RT;
+    constexpr int D = DK * 32, V = VT * 16;
+    constexpr int KP = D * 2 + 16, VP = 80;
+    constexpr int K16 = 32 * (D / 8), V16 = V * 4;
+    constexpr int KPT = (K16 + 255) / 256, VPT = (V16 + 255) / 256;
+    __shared__ __attribute__((aligned(16))) char k_s[32 * KP];
+    __shared__ __attribute__((aligned(16))) char v_s[V * VP];
+    const int e = blockIdx.y, h = blockIdx.z;
+    const int count = p.ent_count[e];
+    if (count < min_count)
+        return;
+    const int tile = (count + ROWS - 1) / ROWS - 1 - (int) blockIdx.x;
+    if (tile < 0)
+        return;
+    const int first = p.ent_first[e], pos0 = p.ent_pos0[e];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int col = lane & 15, g4 = lane >> 4;
+    const int g = h / (p.heads / p.kv_heads);
+    const int page = p.page;
+    const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
+    const HeadMods hm = head_mods(p, h);
+    const uint16_t* kp = reinterpret_cast<const uint16_t*>(p.k_pool);
+    const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.v_pool);
+
+    int r0[RT], qpos[RT], klo[RT], my_blk[RT], my_lo[RT], klo_last[RT];
+    bool rows_ok[RT];
+    bf16x8 qf[RT][DK];
+    float m_run[RT], l_run[RT];
+    f32x4 acc[RT][VT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+    {
+        r0[rt] = tile * ROWS + (w * RT + rt) * 16;
+        rows_ok[rt] = r0[rt] < count; // wave-uniform
+        const int qrow = r0[rt] + col < count ? r0[rt] + col : count - 1;
+        qpos[rt] = pos0 + qrow;
+        klo[rt] = first_visible(p, qpos[rt]);
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks)
+            qf[rt][ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
+                reinterpret_cast<const uint16_t*>(p.q) + ((int64_t) (first + qrow) * p.heads + h) * D + ks * 32 + 8 * g4));
+        const int my_last = r0[rt] + 15 < count ? r0[rt] + 15 : count - 1;
+        my_blk[rt] = rows_ok[rt] ? (pos0 + my_last) / 32 : -1;
+        my_lo[rt] = rows_ok[rt] ? first_visible(p, pos0 + r0[rt]) / 32 : 0;
+        klo_last[rt] = rows_ok[rt] ? first_visible(p, pos0 + my_last) : 0;
+        m_run[rt] = -INFINITY;
+        l_run[rt] = 0.f;
+#pragma unroll
+        for (int ct = 0; ct < VT; ++ct)
+            acc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    const int wg_last = tile * ROWS + ROWS - 1 < count ? tile * ROWS + ROWS - 1 : count - 1;
+    const int nblk = (pos0 + wg_last) / 32 + 1;
+    const int wg_lo = first_visible(p, pos0 + tile * ROWS) / 32;
+
+    uint4 kr[KPT], vr[VPT];
+    int blk_next = table[wg_lo * 32 / page];
+    auto request = [&](int kb) {
+        const int key0 = kb * 32;
+        const int blk = blk_next, off = key0 % page;
+        blk_next = table[kb + 1 < nblk ? (key0 + 32) / page : key0 / page];
+#pragma unroll
+        for (int i = 0; i < KPT; ++i)
+        {
+            const int idx = tid + i * 256;
+            if (K16 % 256 == 0 || idx < K16)
+            {
+                const int row = idx / (D / 8), piece = idx % (D / 8);
+                kr[i] = *reinterpret_cast<const uint4*>(kp + (((int64_t) blk * p.kv_heads + g) * page + off + row) * D + piece * 8);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; ++i)
+        {
+            const int idx = tid + i * 256;
+            if (V16 % 256 == 0 || idx < V16)
+                vr[i] = *reinterpret_cast<const uint4*>(vp + (((int64_t) blk * p.kv_heads + g) * V + idx / 4) * page + off + (idx % 4) * 8);
+        }
+    };
+    request(wg_lo);
+    for (int kb = wg_lo; kb < nblk; ++kb)
+    {
+#pragma unroll
+        for (int i = 0; i < KPT; ++i)
+        {
+            const int idx = tid + i * 256;
+            if (K16 % 256 == 0 || idx < K16)
+                *reinterpret_cast<uint4*>(k_s + (idx / (D / 8)) * KP + (idx % (D / 8)) * 16) = kr[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; ++i)
+        {
+            const int idx = tid + i * 256;
+            if (V16 % 256 == 0 || idx < V16)
+                *reinterpret_cast<uint4*>(v_s + (idx / 4) * VP + (idx % 4) * 16) = vr[i];
+        }
+        __syncthreads();
+        if (kb + 1 < nblk)
+            request(kb + 1);
+        bool on[RT]; // wave-uniform
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+            on[rt] = kb <= my_blk[rt] && kb >= my_lo[rt];
+        if (on[0] || on[RT - 1])
+        {
+            const int key0 = kb * 32;
+            f32x4 s[RT][2];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int ks = 0; ks < DK; ++ks)
+                {
+                    const bf16x8 kfr = as_bf16x8(*reinterpret_cast<const uint4*>(k_s + (t * 16 + col) * KP + (ks * 32 + 8 * g4) * 2));
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+                        if (on[rt])
+                            s[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kfr, qf[rt][ks], s[rt][t], 0, 0, 0);
+                }
+            uint4 pf[RT];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+            {
+                pf[rt] = make_uint4(0, 0, 0, 0);
+                if (on[rt])
+                {
+                    const bool masked = key0 + 31 > pos0 + r0[rt] || key0 < klo_last[rt];
+                    pf[rt] = softmax_block<VT>(s[rt], m_run[rt], l_run[rt], acc[rt], hm, masked, key0 + 4 * g4, qpos[rt], klo[rt]);
+                }
+            }
+#pragma unroll
+            for (int ct = 0; ct < VT; ++ct)
+            {
+                const char* vrow = v_s + (ct * 16 + col) * VP + 8 * g4;
+                const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+                const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 32);
+                const bf16x8 vf = as_bf16x8(make_uint4(lo.x, lo.y, hi.x, hi.y));
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    if (on[rt])
+                        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, as_bf16x8(pf[rt]), acc[rt][ct], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+    {
+        if (!rows_ok[rt] || r0[rt] + col >= count)
+            continue;
+        const float mul = finish_factor(p, h, m_run[rt], l_run[rt]) * out_gate_of(p, first + r0[rt] + col, h);
+        uint16_t* out = reinterpret_cast<uint16_t*>(p.out) + ((int64_t) (first + r0[rt] + col) * p.heads + h) * V + 4 * g4;
+#pragma unroll
+        for (int ct = 0; ct < VT; ++ct)
+            *reinterpret_cast<uint2*>(out + ct * 16)
+                = make_uint2((uint32_t) f2bf(acc[rt][ct][0] * mul) | ((uint32_t) f2bf(acc[rt][ct][1] * mul) << 16),
+                    (uint32_t) f2bf(acc[rt][ct][2] * mul) | ((uint32_t) f2bf(acc[rt][ct][3] * mul) << 16));
+    }
+}
+
 // Second pass of the key split: one wave per (row, head) combines the ks partials of each map, then the differential combination,
 // the head norm and the bfloat16 store.
 template <int MAPS>
@@ -696,8 +864,27 @@ int launch_tile(const StackAttnParams& p, hipStream_t stream)
     const int small_rows = p.max_count < PREFILL_ROWS ? p.max_count : (p.tokens > p.max_count ? PREFILL_ROWS - 1 : 0);
     if (p.max_count >= PREFILL_ROWS)
     {
-        const dim3 pg((p.max_count + 63) / 64, p.entries, p.heads);
-        hipLaunchKernelGGL((attn_prefill_kernel<MAPS, DK, VT>), pg, dim3(256), 0, stream, p, PREFILL_ROWS);
+        // the wide form (128 rows per workgroup) where it still fills the chip; otherwise twice as many workgroups of 64 rows
+        bool wide = false;
+        if constexpr (MAPS == 1 && DK >= 5)
+        {
+            const char* force = std::getenv("TLLM_STACK_WIDE_PREFILL"); // test / measurement knob: 1 = always, 0 = never
+            wide = !p.head_norm
+                && (force ? force[0] == '1' : (int64_t) ((p.max_count + 127) / 128) * p.entries * p.heads >= launch_util::device_cus());
+        }
+        if constexpr (MAPS == 1 && DK >= 5)
+        {
+            if (wide)
+            {
+                const dim3 pg((p.max_count + 127) / 128, p.entries, p.heads);
+                hipLaunchKernelGGL((attn_prefill_wide_kernel<DK, VT>), pg, dim3(256), 0, stream, p, PREFILL_ROWS);
+            }
+        }
+        if (!wide)
+        {
+            const dim3 pg((p.max_count + 63) / 64, p.entries, p.heads);
+            hipLaunchKernelGGL((attn_prefill_kernel<MAPS, DK, VT>), pg, dim3(256), 0, stream, p, PREFILL_ROWS);
+        }
     }
     if (small_rows > 0)
     {

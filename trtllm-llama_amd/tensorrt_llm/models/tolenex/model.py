@@ -8,14 +8,11 @@ This class reads the model's config.json and its safetensors file and describes 
 (runtime/stack.py); there is no Python forward pass.  Constants the design fixes live here (two maps per attention head, the
 head norm, gelu-tanh in the feed-forward, the gated residual); everything else is read from the configuration."""
 import json
-import os
 from typing import Dict
 
 import numpy as np
 
-from ..._utils import read_safetensors
-
-PAGE_SIZE = 64
+from ..stack_model import PAGE_SIZE, StackModelForCausalLM, bf16_bits_to_f32, to_bf16_bits  # noqa: F401
 
 
 class TolenexConfig(object):
@@ -70,18 +67,9 @@ class TolenexConfig(object):
         return c
 
 
-class TolenexForCausalLM(object):
+class TolenexForCausalLM(StackModelForCausalLM):
     architecture = 'Tolenex'
-    page_size = PAGE_SIZE
-
-    def __init__(self, config: TolenexConfig, tensors: Dict):
-        self.config, self.tensors = config, tensors
-
-    @classmethod
-    def from_checkpoint(cls, model_dir: str) -> 'TolenexForCausalLM':
-        """model_dir: config.json + model.safetensors (bfloat16 weights, linear weights [out, in])."""
-        config = TolenexConfig.from_json_file(os.path.join(model_dir, 'config.json'))
-        return cls(config, read_safetensors(os.path.join(model_dir, 'model.safetensors')))
+    config_class = TolenexConfig
 
     @classmethod
     def from_random(cls, config: Dict, seed: int = 0, std: float = 0.02) -> 'TolenexForCausalLM':
@@ -130,22 +118,3 @@ class TolenexForCausalLM(object):
                 mat(p + 'mlp.up', F, W, s=W ** -0.5)
                 mat(p + 'mlp.down', W, F, s=F ** -0.5)
         return cls(cfg, t)
-
-    def build_stack_engine(self, dtype: str = 'bfloat16', num_blocks: int = 64, num_slots: int = 4, debug_taps: bool = False,
-                           build_if_missing: bool = False):
-        from ...runtime.stack import StackEngine
-        if dtype not in ('bfloat16', 'float32'):
-            raise ValueError(f'dtype {dtype!r}: bfloat16 or float32')
-        c = self.config.engine_config()
-        c.update(dtype=dtype, num_blocks=num_blocks, num_slots=num_slots, debug_taps=int(debug_taps))
-        return StackEngine(c, self.tensors, build_if_missing=build_if_missing)
-
-
-def to_bf16_bits(a: np.ndarray) -> np.ndarray:
-    """fp32 array -> bfloat16 bit patterns (uint16), round to nearest even."""
-    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
-    return ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16).reshape(a.shape)
-
-
-def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
-    return (b.astype(np.uint32) << 16).view(np.float32)

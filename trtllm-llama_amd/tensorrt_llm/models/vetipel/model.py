@@ -58,7 +58,8 @@ class VetipelConfig(object):
             c[p + 'heads'], c[p + 'dim'], c[p + 'vdim'] = int(m['heads']), int(m['dim']), int(m.get('vdim', m['dim']))
             c[p + 'ff'] = int(l['mlp']['ff']) if l.get('mlp') else 0
             c[p + 'mlp'] = 'relu2'
-            c[p + 'scale'] = repr(float(m['scale']))
+            if 'scale' in m:     # absent: the engine's default, 1 / sqrt(query size)
+                c[p + 'scale'] = repr(float(m['scale']))
             if l['type'] == 'latent_attention':
                 c[p + 'type'] = 'latent_attention'
                 c[p + 'kv_rank'] = int(m['kv_rank'])
@@ -71,13 +72,14 @@ class VetipelConfig(object):
             c[p + 'kv_heads'] = int(m.get('kv_heads', m['heads']))
             c[p + 'maps'], c[p + 'head_norm'], c[p + 'rot_dims'] = 1, 0, 0
             c[p + 'out_gate'] = 1
-            c[p + 'mask_size'] = int(m['mask']['size'])
+            size = int((m.get('mask') or {}).get('size', 0))   # no size: plain causal
+            c[p + 'mask_size'] = size
             if l['type'] == 'attention':
                 c[p + 'pos_bias'], c[p + 'slope_base'] = 'linear', repr(SLOPE_BASE)
-                c[p + 'mask'], c[p + 'weights'] = 'window', 'sigmoid'
+                c[p + 'mask'], c[p + 'weights'] = ('window' if size else 'causal'), 'sigmoid'
             else:
                 c[p + 'qkv_bias'], c[p + 'qk_norm'], c[p + 'head_temp'], c[p + 'sink'] = 1, 1, 1, 1
-                c[p + 'pos_bias'], c[p + 'mask'], c[p + 'weights'] = 'log', 'chunk', 'softmax'
+                c[p + 'pos_bias'], c[p + 'mask'], c[p + 'weights'] = 'log', ('chunk' if size else 'causal'), 'softmax'
         return c
 
 
