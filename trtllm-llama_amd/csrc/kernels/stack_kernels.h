@@ -72,7 +72,8 @@ int launch_stack_group_rmsnorm(void* y1, void* y2, const float* x, const int32_t
 //   2. u = sum_s in[s] xs[s]  (in == null: the plain sum)
 //   3. h != null: h = u / sqrt(mean(u^2) + eps) * w   (element type `dtype`: the next sublayer's input)
 //      sum_out != null: sum_out = u (fp32)
-// Everything is fp32 but h.  mix / out / in are device arrays.
+// rows (optional gather): launch row r works on packed row rows[r] and writes h row r - the last reader of the streams (the output
+// norm) only touches the rows whose logits are wanted, and writes nothing back into the streams.  Everything is fp32 but h.  mix / out / in are device arrays.
 struct StackHyperParams
 {
     int32_t dtype = DT_BF16;
@@ -87,6 +88,7 @@ struct StackHyperParams
     const float* w = nullptr;   // [width] norm weight as applied (any offset already added)
     float eps = 1e-5f;
     float* sum_out = nullptr;
+    const int32_t* rows = nullptr; // [tokens] or null
 };
 int launch_stack_hyper_norm(const StackHyperParams& p, hipStream_t stream);
 // y[t, c] = gelu_tanh(gu[t, c]) * gu[t, ff + c] over a [tokens, ld] projection that holds gate then up columns

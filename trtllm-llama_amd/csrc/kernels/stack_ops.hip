@@ -92,7 +92,7 @@ __global__ __launch_bounds__(HY_T) void hyper_norm_kernel(const StackHyperParams
     extern __shared__ float u_s[]; // [width]
     __shared__ float red[32];
     __shared__ float cm[HY_MAXS * HY_MAXS], co[HY_MAXS], ci[HY_MAXS];
-    const int t = blockIdx.x, tid = threadIdx.x, S = p.streams;
+    const int t = p.rows ? p.rows[blockIdx.x] : blockIdx.x, tid = threadIdx.x, S = p.streams;
     if (tid < S * S)
         cm[tid] = p.y ? p.mix[tid] : 0.f;
     if (tid < S)
@@ -123,7 +123,8 @@ __global__ __launch_bounds__(HY_T) void hyper_norm_kernel(const StackHyperParams
                         if (s < S)
                             a = fmaf(cm[s * S + to], xs[s], a);
                     a = fmaf(co[to], y, a);
-                    p.x[to * p.stream_stride + o] = a;
+                    if (!p.rows) // a gathered launch is the streams' last reader (and a row may be asked for twice): nothing is written back
+                        p.x[to * p.stream_stride + o] = a;
                     u = fmaf(ci[to], a, u);
                 }
             }
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(HY_T) void hyper_norm_kernel(const StackHyperParams
     ss = block_sum(ss, red);
     const float inv = 1.f / sqrtf(ss / (float) p.width + p.eps);
     for (int c = tid; c < p.width; c += HY_T)
-        El<DT>::st(p.h, (int64_t) t * p.width + c, u_s[c] * inv * p.w[c]);
+        El<DT>::st(p.h, (int64_t) blockIdx.x * p.width + c, u_s[c] * inv * p.w[c]);
 }
 
 __global__ __launch_bounds__(256) void pass_entry_kernel(float* x, const float* add, const float* row, int64_t n, int width)
@@ -836,7 +837,7 @@ template <int DT, int SM>
 __global__ __launch_bounds__(1024) void hyper_norm_vec_kernel(const StackHyperParams p)
 {
     __shared__ float red[32];
-    const int t = blockIdx.x, tid = threadIdx.x, S = p.streams, W4 = p.width >> 2, NT = blockDim.x;
+    const int t = p.rows ? p.rows[blockIdx.x] : blockIdx.x, tid = threadIdx.x, S = p.streams, W4 = p.width >> 2, NT = blockDim.x;
     float4 xs[HV_K][SM], yv[HV_K], u[HV_K];
 #pragma unroll
     for (int k = 0; k < HV_K; ++k)
@@ -885,7 +886,7 @@ __global__ __launch_bounds__(1024) void hyper_norm_vec_kernel(const StackHyperPa
                 n.y = fmaf(co[to], yv[k].y, n.y);
                 n.z = fmaf(co[to], yv[k].z, n.z);
                 n.w = fmaf(co[to], yv[k].w, n.w);
-                if (to < S && c4 < W4)
+                if (to < S && c4 < W4 && !p.rows) // a gathered launch is the streams' last reader: nothing is written back
                     reinterpret_cast<float4*>(p.x + to * p.stream_stride + (int64_t) t * p.width)[c4] = n;
             }
             acc.x = fmaf(ci[to], n.x, acc.x);
@@ -909,7 +910,7 @@ __global__ __launch_bounds__(1024) void hyper_norm_vec_kernel(const StackHyperPa
         if (c4 < W4)
         {
             const float4 w = reinterpret_cast<const float4*>(p.w)[c4];
-            const int64_t o = (int64_t) t * p.width + 4 * c4;
+            const int64_t o = (int64_t) blockIdx.x * p.width + 4 * c4;
             if (DT == DT_BF16)
                 *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.h) + o)
                     = make_uint2((uint32_t) f2bf(u[k].x * inv * w.x) | ((uint32_t) f2bf(u[k].y * inv * w.y) << 16),

@@ -1160,17 +1160,32 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         if (s->taps)
             HIP_OK(hipMemcpyAsync(s->tap + ri * (size_t) T * Wd, s->x, (size_t) T * Wd * 4, hipMemcpyDeviceToDevice, stream));
     }
-    // the row the final norm reads: the sum of the streams (one stream of the gated residual: x itself)
-    const float* x_final = s->x;
-    if (s->hyper)
-    {
-        if (hyper(nullptr, nullptr, nullptr, s->x0))
-            return -1;
-        x_final = s->x0;
-    }
     if (NW > 0)
     {
-        if (launch_stack_group_rmsnorm(s->hw, nullptr, x_final, d_want, s->final_norm, nullptr, s->dtype, NW, Wd, s->groups, s->eps, stream))
+        if (s->hyper)
+        {
+            // the output norm reads the sum of the streams; the last sublayer lands in the same launch, on the wanted rows only
+            StackHyperParams hp;
+            hp.dtype = s->dtype;
+            hp.tokens = NW;
+            hp.width = Wd;
+            hp.streams = s->streams;
+            hp.x = s->x;
+            hp.stream_stride = stream_stride;
+            if (pending)
+            {
+                hp.y = s->y32;
+                hp.mix = pending->mix;
+                hp.out = pending->out;
+            }
+            hp.h = s->hw;
+            hp.w = s->final_norm;
+            hp.eps = s->eps;
+            hp.rows = d_want;
+            if (launch_stack_hyper_norm(hp, stream))
+                return -1;
+        }
+        else if (launch_stack_group_rmsnorm(s->hw, nullptr, s->x, d_want, s->final_norm, nullptr, s->dtype, NW, Wd, s->groups, s->eps, stream))
             return -1;
         StackGemmParams hd;
         hd.dtype = s->dtype;
