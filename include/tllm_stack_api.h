@@ -11,9 +11,14 @@
  *
  * Mixer kinds: "attention" (grouped-query, `maps` attention maps per head over shared values - 2 = differential attention -,
  * interleaved rotary positions on the first rot_dims dimensions with YaRN-style frequency scaling, tanh soft cap, per-head RMS
- * norm of the output) and "hgrn2" (gated linear recurrence with a lower-bounded forget gate, fp32 state).  Norms are RMS norms in
- * groups; residual updates are gated by sigmoid(W h + b); a range of layers may be run several times in a row (every pass with a
- * cache / state of its own).
+ * norm of the output; optionally projection biases, unit-RMS queries and keys, a per-head temperature, a linear or logarithmic
+ * distance penalty, a sliding-window or chunked mask, sigmoid weights instead of a softmax, a softmax sink, a per-head output
+ * gate), "latent_attention" (keys and values expanded from one low-rank latent per token plus one rotated key part shared by the
+ * heads; the cache holds the latent and that part, attention runs in the absorbed form) and "hgrn2" (gated linear recurrence with
+ * a lower-bounded forget gate, fp32 state).  Two block forms: parallel sublayers on one residual whose updates are gated by
+ * sigmoid(W h + b), RMS norms in groups, a range of layers optionally run several times in a row (every pass with a cache / state
+ * of its own); or sequential pre-norm sublayers on `streams` hyper-connected residual copies (u = sum_s in[s] x_s feeds the
+ * sublayer, x_t <- sum_s mix[s, t] x_s + out[t] y lands its result; the output norm reads sum_s x_s).
  *
  * Element type bfloat16: weights, activations and caches in bfloat16, fp32 accumulation, and fp32 for the residual stream, norms,
  * scores and softmax, rotation angles, gates of a recurrence and its state.  float32: everything in fp32 with plain FMAs.
@@ -35,13 +40,20 @@ typedef struct tllm_stack* tllm_stack_t;
 /* Configuration text, one key=value per line:
  *   dtype (bfloat16 | float32), width, vocab, num_layers, norm_groups (1), norm_eps (1e-5), embedding_scale (1),
  *   loop_start, loop_stop, loop_times (0, 0, 1: no loop), page_size (64), num_blocks, num_slots, debug_taps (0),
- *   per layer i: layer.<i>.type (attention | hgrn2), .heads, .dim, .vdim, .ff (0: no feed-forward),
+ *   block (parallel | sequential), residual (gated | hyper; parallel goes with gated, sequential with hyper), streams (1 .. 8),
+ *   norm_offset (0: a norm weight is applied as norm_offset + stored value),
+ *   per layer i: layer.<i>.type (attention | latent_attention | hgrn2), .heads, .dim, .vdim, .ff (0: no feed-forward),
+ *     .mlp (gelu_gate: W_down (gelu_tanh(W_gate h) * W_up h) | relu2: W_down relu(W_up h)^2, sequential blocks only),
  *     attention: .kv_heads, .maps (1 | 2), .diff (the constant of the second map's weight and of the output scale 1 - diff),
  *       .scale, .softcap (0: none), .head_norm (0 | 1), .rot_dims, .rot_base, .rot_factor (0: no frequency scaling),
- *       .rot_original, .rot_fast, .rot_slow.
- * Weights are named l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,lq1,lk1,lq2,lk2} (attention), l<i>.mix.{q,f,f.b,lower,v,norm,o}
- * (hgrn2), l<i>.mlp.{gate,up,down}, l<i>.rg1, l<i>.rg1.b, l<i>.rg2, l<i>.rg2.b, embed, loop.step, final.norm, head; linear
- * weights [out, in]. */
+ *       .rot_original, .rot_fast, .rot_slow, .qkv_bias (0 | 1), .qk_norm (0 | 1: q and k / their RMS over dim), .head_temp (0 | 1),
+ *       .pos_bias (none | linear: slope_h = 2^(-slope_base (h + 1) / heads) | log: r1_h ln(1 + r2_h (i - j))), .slope_base (8),
+ *       .mask (causal | window | chunk), .mask_size, .weights (softmax | sigmoid), .sink (0 | 1), .out_gate (0 | 1);
+ *     latent_attention: .kv_rank, .rot_dim (size of the shared rotated part), .rot_dims (how many of them turn), .rot_base, .scale.
+ * Weights are named l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,lq1,lk1,lq2,lk2} (attention; with the options also q.b, k.b, v.b,
+ * temp, r1, r2, sink, pb, g), l<i>.mix.{q,dkv,dkv.norm,uk,uv,o} (latent_attention), l<i>.mix.{q,f,f.b,lower,v,norm,o} (hgrn2),
+ * l<i>.mlp.{gate,up,down}, l<i>.rg1, l<i>.rg1.b, l<i>.rg2, l<i>.rg2.b (gated residual), l<i>.hc{1,2}.{in,out,mix} (hyper
+ * residual; absent with one stream: the plain sum), embed, loop.step, final.norm, head; linear weights [out, in]. */
 tllm_stack_t tllm_stack_create(const char* config_text);
 
 /* One weight tensor from HOST memory; dtype 0 = fp32, 7 = bfloat16 (nvinfer1::DataType codes).  Converted to the engine's element
@@ -77,7 +89,8 @@ int64_t tllm_stack_weight_bytes(tllm_stack_t s);
 /* bytes one step moves at least: weights once, plus the cache / state the given contexts touch (roofline denominators) */
 int64_t tllm_stack_step_bytes(tllm_stack_t s, int32_t n_tokens, int64_t context_tokens, int32_t n_entries);
 
-/* debug_taps=1: the residual stream behind layer run `run` of the last step, fp32 [n_tokens, width], to host memory. */
+/* debug_taps=1: the residual stream behind layer run `run` of the last step (the sum of the streams, if there are several), fp32
+ * [n_tokens, width], to host memory. */
 int32_t tllm_stack_get_tap(tllm_stack_t s, int32_t run, float* out, size_t n_floats);
 
 void tllm_stack_destroy(tllm_stack_t s);

@@ -73,6 +73,8 @@ MECHANISMS = {
     'whole_stack': make_config(FULL, emb_scale=1.0, eps=3e-6),
     'tiled_stack': make_config(TILED, streams=2),
     'width_that_is_no_multiple_of_four': make_config([window_layer(ff=30), latent_layer(ff=0), chunk_layer(ff=22)], width=70, vocab=131, streams=2),
+    'odd_head_sizes': make_config([window_layer(heads=3, kv_heads=1, dim=9, vdim=7, size=11, ff=30), chunk_layer(heads=2, kv_heads=2, dim=5, vdim=3, size=9),
+                                   latent_layer(heads=2, dim=7, rot_dim=6, vdim=5, kv_rank=13, ff=0)], width=52, vocab=131, streams=2),
     'wide_values': make_config([window_layer(heads=2, kv_heads=1, dim=8, vdim=160, size=20)]),
 }
 

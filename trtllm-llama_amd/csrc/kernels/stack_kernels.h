@@ -1,6 +1,7 @@
 // Host-side launch interface of the kernels behind the ragged-batch stack engine (runtime/stack_engine.cpp): decoder
-// stacks whose layers are described at run time (grouped RMS norms, gated residuals, looped layer ranges, differential
-// attention over a paged cache, HGRN2 recurrences over per-sequence state slots).
+// stacks whose layers are described at run time (grouped RMS norms, gated residuals or hyper-connected residual streams, looped
+// layer ranges, attention over a paged cache in its variants - differential maps, masks, distance penalties, sigmoid weights, sinks,
+// a shared latent -, HGRN2 recurrences over per-sequence state slots).
 //
 // A step is one packed batch of `tokens` rows: portions of prompts and single decoded tokens of several sequences side
 // by side.  Row t belongs to batch entry tok_entry[t] and sits at position tok_pos[t] of its sequence.  Every kernel is

@@ -1024,9 +1024,9 @@ static bool attn_shape_ok(const StackAttnParams& p, const char* what)
             p.kv_heads, p.maps, p.dim, p.vdim, p.page, p.max_blocks);
         return false;
     }
-    if ((p.dim & 1) || (p.rot_dims & 1) || p.rot_dims > p.dim || p.rot_dims < 0)
+    if ((p.rot_dims & 1) || p.rot_dims > p.dim || p.rot_dims < 0)
     {
-        set_error("%s: the rotation pairs neighbours: dim %d and rot_dims %d must be even, rot_dims <= dim", what, p.dim, p.rot_dims);
+        set_error("%s: the rotation pairs neighbours: rot_dims %d must be even and <= dim %d", what, p.rot_dims, p.dim);
         return false;
     }
     if (p.mask < MASK_CAUSAL || p.mask > MASK_CHUNK || (p.mask != MASK_CAUSAL && p.mask_size < 1) || p.weights < WEIGHTS_SOFTMAX
@@ -1044,6 +1044,11 @@ int launch_stack_rope_kv(const StackAttnParams& p, hipStream_t stream)
         return 0;
     if (!attn_shape_ok(p, "stack_rope_kv"))
         return -1;
+    if (p.rot_dims > 0 && (p.dim & 1))
+    {
+        set_error("stack_rope_kv: the rotation pairs (2i, 2i + 1) inside every head: dim %d must be even", p.dim);
+        return -1;
+    }
     if (p.bias || p.qk_unit_norm)
     {
         if (p.dim > 64 * PREP_EPL)

@@ -402,8 +402,8 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.rot_dims = geti(s, p + "rot_dims", l.rot_part);
             l.rot_base = getd(s, p + "rot_base", 10000);
             l.scale = getd(s, p + "scale", 1.0 / std::sqrt((double) (l.dim + l.rot_part)));
-            if (l.kv_rank < 1 || l.rot_part < 0 || l.rot_dims < 0 || (l.rot_dims & 1) || l.rot_dims > l.rot_part || ((l.kv_rank + l.rot_part) & 1))
-                return fail("latent_attention: kv_rank positive, rot_dims even and <= rot_dim, kv_rank + rot_dim even");
+            if (l.kv_rank < 1 || l.rot_part < 0 || l.rot_dims < 0 || (l.rot_dims & 1) || l.rot_dims > l.rot_part)
+                return fail("latent_attention: kv_rank positive, rot_dims even and <= rot_dim");
             l.kv_heads = 1;
             l.n_q = l.heads * (l.dim + l.rot_part);
             l.n_k = l.kv_rank + l.rot_part; // the down projection: latent | rotated key part
@@ -445,8 +445,9 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.rot_original = getd(s, p + "rot_original", 0);
             l.rot_fast = getd(s, p + "rot_fast", 0);
             l.rot_slow = getd(s, p + "rot_slow", 0);
-            if (l.kv_heads < 1 || l.heads % l.kv_heads || l.maps < 1 || l.maps > 2 || (l.dim & 1) || (l.rot_dims & 1) || l.rot_dims > l.dim)
-                return fail("attention: heads must be a multiple of kv_heads, maps 1 or 2, dim and rot_dims even, rot_dims <= dim");
+            if (l.kv_heads < 1 || l.heads % l.kv_heads || l.maps < 1 || l.maps > 2 || (l.rot_dims > 0 && (l.dim & 1)) || (l.rot_dims & 1)
+                || l.rot_dims > l.dim)
+                return fail("attention: heads must be a multiple of kv_heads, maps 1 or 2, rot_dims even and <= dim, dim even where anything turns");
             l.n_q = l.heads * l.maps * l.dim;
             l.n_k = l.kv_heads * l.maps * l.dim;
             l.n_v = l.kv_heads * l.vdim;
