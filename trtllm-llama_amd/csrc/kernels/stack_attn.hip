@@ -972,7 +972,11 @@ int launch_stack_attention(const StackAttnParams& p, hipStream_t stream)
 {
     if (p.tokens <= 0)
         return 0;
-    if (p.heads >= 1 && p.kv_heads >= 1 && p.heads % p.kv_heads == 0 && stack_attention_tiled(p))
+    static const bool general_only = [] {
+        const char* v = std::getenv("TLLM_STACK_ATTN_GENERAL"); // measurement knob: 1 = every shape on the general kernel
+        return v && v[0] == '1';
+    }();
+    if (!general_only && p.heads >= 1 && p.kv_heads >= 1 && p.heads % p.kv_heads == 0 && stack_attention_tiled(p))
     {
         int rc = p.maps == 2 ? launch_tile_d<2>(p, stream) : (p.maps == 1 ? launch_tile_d<1>(p, stream) : 1);
         if (rc == 1 && p.maps == 1)
