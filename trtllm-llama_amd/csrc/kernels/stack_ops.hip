@@ -828,6 +828,8 @@ int launch_stack_embed(float* x, float* keep, const int32_t* ids, const void* ta
     return launched("stack_embed");
 }
 
+namespace
+{
 // The form for rows of a multiple of 4 up to HV_K * 4096 elements: up to 1024 threads, a thread owns HV_K float4 columns of every
 // stream and has ALL of them in flight before its first store (the streams are read and written through the same pointer, so in
 // a loop every store would fence the loads behind it); the combined row stays in registers.
@@ -923,7 +925,7 @@ __global__ __launch_bounds__(1024) void hyper_norm_vec_kernel(const StackHyperPa
 }
 
 template <int DT>
-static void launch_hyper_vec(const StackHyperParams& p, int nt, hipStream_t stream)
+void launch_hyper_vec(const StackHyperParams& p, int nt, hipStream_t stream)
 {
     if (p.streams <= 1)
         hipLaunchKernelGGL((hyper_norm_vec_kernel<DT, 1>), dim3(p.tokens), dim3(nt), 0, stream, p);
@@ -934,6 +936,8 @@ static void launch_hyper_vec(const StackHyperParams& p, int nt, hipStream_t stre
     else
         hipLaunchKernelGGL((hyper_norm_vec_kernel<DT, 8>), dim3(p.tokens), dim3(nt), 0, stream, p);
 }
+
+} // namespace
 
 int launch_stack_hyper_norm(const StackHyperParams& p, hipStream_t stream)
 {
